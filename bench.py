@@ -1,0 +1,159 @@
+#!/usr/bin/env python3
+"""Benchmark of the per-thread forward+backward hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A step is one pass of the forward+backward kernels over the whole batch of
+synthetic problems (N = 64 Mi, inputs already resident in HBM).  Prints one JSON
+line: throughput in evaluations per second, the HBM roofline of the kernel
+(algorithmic bytes = 52 B per evaluation) and a CPU baseline measured in the
+same run on the host cores.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published
+N_FULL = 64 * 1024 * 1024
+
+
+def cpu_baseline(host_inputs, budget_s=12.0):
+    """Times the CPU oracle (the reference's formulas restated in C, OpenMP over
+    all host cores the box gives us) on a bounded sample of the same workload."""
+    import numpy as np
+
+    from tests import _oracle
+
+    oracle = _oracle.load()
+    cores = min(oracle.max_threads(), int(os.environ.get("OMP_NUM_THREADS", "0") or 0) or oracle.max_threads())
+    oracle.set_threads(cores)
+    n = host_inputs[0].size
+    oracle.chain_soa(host_inputs, np.float32)  # warm-up
+    reps, t0 = 0, time.perf_counter()
+    while True:
+        oracle.chain_soa(host_inputs, np.float32)
+        reps += 1
+        dt = time.perf_counter() - t0
+        if dt >= budget_s:
+            break
+    return {
+        "value": n * reps / dt,
+        "unit": "evals/s",
+        "cores": cores,
+        "kind": "port",
+        "sample": "first %d problems of the workload, %d passes, %.1f s" % (n, reps, dt),
+    }
+
+
+def host_templates(host_inputs):
+    """The library's own templates compiled for the host cores (N = 1e6)."""
+    import numpy as np
+
+    from xyz_autodiff_cuda_amd import chain
+
+    threads = int(os.environ.get("OMP_NUM_THREADS", "0") or 0) or (os.cpu_count() or 1)
+    sample = [a[:1_000_000] for a in host_inputs]
+    chain.host_forward_backward(sample, np.float32, threads)
+    best = float("inf")
+    for _ in range(10):
+        t0 = time.perf_counter()
+        chain.host_forward_backward(sample, np.float32, threads)
+        best = min(best, time.perf_counter() - t0)
+    n = sample[0].size
+    return {"value": n / best, "unit": "evals/s", "threads": threads, "n": n, "GBps": 52.0 * n / best / 1e9}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--n", type=int, default=N_FULL, help="problems per step (default: the full 64 Mi)")
+    ap.add_argument("--seed", type=int, default=1234)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs (profiling runs)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this build has no multi-GPU path (got --gpus %d)" % args.gpus)
+
+    import numpy as np
+    import torch
+
+    from xyz_autodiff_cuda_amd import chain, rng
+
+    assert torch.cuda.is_available(), "bench.py needs the GPU"
+    dev = torch.device("cuda:0")
+    n = args.n
+    ins = [torch.empty(n, dtype=torch.float32, device=dev) for _ in range(6)]
+    outs = [torch.empty(n, dtype=torch.float32, device=dev) for _ in range(7)]
+    rng.chain_inputs_(ins, args.seed)
+    torch.cuda.synchronize()
+
+    for _ in range(args.warmup):
+        chain.forward_backward(ins, outs)
+    torch.cuda.synchronize()
+
+    starts = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps)]
+    stops = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for k in range(args.steps):
+        starts[k].record()
+        chain.forward_backward(ins, outs)
+        stops[k].record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+
+    kernel_ms = [a.elapsed_time(b) for a, b in zip(starts, stops)]
+    avg_kernel_s = sum(kernel_ms) / len(kernel_ms) / 1e3
+    algorithmic_bytes = float(chain.BYTES_PER_EVAL) * n
+    achieved = algorithmic_bytes / avg_kernel_s / 1e9
+
+    finite = all(bool(torch.isfinite(o).all()) for o in outs)
+
+    record = {
+        "metric": "per-thread fwd+bwd evals/sec",
+        "value": n * args.steps / wall,
+        "unit": "evals/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": wall / args.steps * 1e3,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {
+            "workload": "config 2: per-thread forward+backward chain, N=%d, fp32, SoA (6 in, 7 out), seed %d" % (n, args.seed),
+            "n": n,
+            "bytes_per_eval": chain.BYTES_PER_EVAL,
+        },
+        "roofline": {
+            "bound": "hbm",
+            "achieved": achieved,
+            "peak": HBM_PEAK_GBPS,
+            "unit": "GB/s",
+            "frac": achieved / HBM_PEAK_GBPS,
+            "traffic": None,
+            "kernel": "chain_quad_kernel",
+            "kernel_ms_avg": avg_kernel_s * 1e3,
+            "kernel_ms_min": min(kernel_ms),
+        },
+        "outputs_finite": finite,
+    }
+    if not args.no_cpu:
+        sample_n = min(n, 8 * 1024 * 1024)
+        host_inputs = [t[:sample_n].cpu().numpy() for t in ins]
+        record["cpu_baseline"] = cpu_baseline(host_inputs)
+        record["host_templates"] = host_templates(host_inputs)
+    print(json.dumps(record))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,100 @@
+/* C ABI of libxad_hip.so: the GPU entry points of the per-thread autodiff hot
+ * path on AMD MI355X (gfx950), plus the host-core build of the same templates.
+ *
+ * xyz-autodiff-cuda has no C ABI, plugin or FFI: its boundary is a C++
+ * template API used inside user kernels (kept, header for header, under
+ * include/xyz_autodiff/).  What a binding would wrap are the kernels and host
+ * launchers that its tests and examples build on top of those templates; each
+ * entry point below names the one it stands in for.
+ *
+ * Conventions
+ *   - every pointer documented as "device" is HBM memory of the current HIP
+ *     device; "host" pointers are ordinary process memory;
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream);
+ *     calls are asynchronous with respect to the host unless stated otherwise;
+ *   - the return value is XAD_OK or one of the XAD_ERR_* codes; the text of the
+ *     last failure on the calling thread is available from xad_last_error().
+ *     (The reference's host helpers throw std::runtime_error instead,
+ *     include/xyz_autodiff/util/error_checker.cuh:9-20.)
+ *   - nothing here falls back to the CPU: an entry point without the xad_host_
+ *     prefix either runs on the GPU or fails.
+ */
+#ifndef XAD_CAPI_H
+#define XAD_CAPI_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define XAD_OK 0
+#define XAD_ERR_INVALID_ARGUMENT 1 /* null pointer, bad size, bad enum value    */
+#define XAD_ERR_HIP 2              /* a HIP runtime call or kernel launch failed */
+#define XAD_ERR_UNSUPPORTED 3      /* valid request this build cannot serve      */
+
+/* Text of the most recent error on this thread ("" if none). */
+const char* xad_last_error(void);
+
+/* ABI revision of this library; bumped on incompatible changes. */
+int xad_abi_version(void);
+
+/* ---------------------------------------------------------------------------
+ * Per-thread forward + backward of the benchmark graph, structure of arrays.
+ *
+ *   es = exp((sx, sy)); Sigma = R(theta) diag(es)^2 R(theta)^T; q = p^T Sigma^-1 p;
+ *   w = sigmoid(o) * exp(-q / 2);   outputs: w and d w / d (sx, sy, theta, o, px, py)
+ *
+ * Six device input arrays and seven device output arrays of n floats each; no
+ * two output arrays may overlap each other or an input.  Arrays aligned to 16
+ * bytes are processed with 16-byte loads and stores (four problems per lane);
+ * any other alignment is served by the 4-byte kernel.  n may be 0.
+ * Stands in for the per-Gaussian graph that gaussian_splatting_kernel builds
+ * and runs per (pixel, Gaussian)
+ * (examples/mini-gaussian-splatting/gaussian_splatting_kernel.cu:73-111) and for
+ * the <<<1,1>>> graph kernels of the reference tests (tests/test_dag_backward.cu:43-67).
+ */
+int xad_chain_forward_backward_f32(size_t n,
+                                   const float* sx, const float* sy, const float* theta,
+                                   const float* o, const float* px, const float* py,
+                                   float* w, float* d_sx, float* d_sy, float* d_theta,
+                                   float* d_o, float* d_px, float* d_py,
+                                   void* stream);
+
+/* The same graph from the same templates, compiled for the host and run on
+ * `num_threads` host threads (<= 0: all hardware threads).  Host pointers.
+ * Synchronous.  This is the "host-core run of the per-thread templates"; GPU
+ * entry points never route through it. */
+int xad_host_chain_forward_backward_f32(size_t n,
+                                        const float* sx, const float* sy, const float* theta,
+                                        const float* o, const float* px, const float* py,
+                                        float* w, float* d_sx, float* d_sy, float* d_theta,
+                                        float* d_o, float* d_px, float* d_py,
+                                        int num_threads);
+int xad_host_chain_forward_backward_f64(size_t n,
+                                        const double* sx, const double* sy, const double* theta,
+                                        const double* o, const double* px, const double* py,
+                                        double* w, double* d_sx, double* d_sy, double* d_theta,
+                                        double* d_o, double* d_px, double* d_py,
+                                        int num_threads);
+
+/* ---------------------------------------------------------------------------
+ * Synthetic inputs: counter-based generator, element i of a fill is a pure
+ * function of (seed, stream_id, i).  The reference seeds std::mt19937 on the
+ * host and uploads (examples/mini-gaussian-splatting/gaussian_parameters.cu:27-66);
+ * these fill device memory in place.
+ */
+int xad_rng_uniform_f32(float* dst, size_t n, uint64_t seed, uint64_t stream_id,
+                        float lo, float hi, void* stream);
+int xad_rng_normal_f32(float* dst, size_t n, uint64_t seed, uint64_t stream_id,
+                       float mean, float stddev, void* stream);
+/* Host: the raw 64 random bits of elements first .. first+n-1. */
+int xad_host_rng_bits(uint64_t* dst, size_t n, uint64_t seed, uint64_t stream_id, uint64_t first);
+int xad_host_rng_uniform_f32(float* dst, size_t n, uint64_t seed, uint64_t stream_id,
+                             float lo, float hi);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* XAD_CAPI_H */

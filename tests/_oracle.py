@@ -1,0 +1,79 @@
+"""ctypes access to oracle/liboracle.so for the tests (the checker side only)."""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+ORACLE_DIR = os.path.join(ROOT, "oracle")
+LIB_PATH = os.path.join(ORACLE_DIR, "liboracle.so")
+
+_lib = None
+
+
+def load():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            subprocess.run(["make", "-C", ORACLE_DIR], check=True, capture_output=True)
+        _lib = ctypes.CDLL(LIB_PATH)
+    return Oracle(_lib)
+
+
+_CT = {np.dtype(np.float32): ctypes.c_float, np.dtype(np.float64): ctypes.c_double}
+_SUF = {np.dtype(np.float32): "_f32", np.dtype(np.float64): "_f64"}
+
+
+def _arg(x, dtype):
+    """numpy array -> pointer, python int -> c_int, python float -> REAL."""
+    if isinstance(x, np.ndarray):
+        assert x.dtype == dtype and x.flags["C_CONTIGUOUS"], (x.dtype, dtype)
+        return x.ctypes.data_as(ctypes.c_void_p)
+    if isinstance(x, (int, np.integer)):
+        return ctypes.c_int(int(x))
+    if isinstance(x, float):
+        return _CT[dtype](x)
+    if x is None:
+        return ctypes.c_void_p(0)
+    raise TypeError(type(x))
+
+
+class Oracle:
+    def __init__(self, lib):
+        self.lib = lib
+
+    def call(self, name, dtype, *args):
+        """Calls oracle_<name>_f32/_f64 with numpy arrays / ints / floats."""
+        dtype = np.dtype(dtype)
+        fn = getattr(self.lib, "oracle_" + name + _SUF[dtype])
+        fn.restype = None
+        fn(*[_arg(a, dtype) for a in args])
+
+    def chain_one(self, inputs, dtype):
+        """inputs = (sx, sy, theta, o, px, py) -> (w, grads[6], q)."""
+        dtype = np.dtype(dtype)
+        x = np.asarray(inputs, dtype=dtype)
+        w = np.zeros(1, dtype)
+        g = np.zeros(6, dtype)
+        q = np.zeros(1, dtype)
+        self.call("chain_one", dtype, x, w, g, q)
+        return w[0], g, q[0]
+
+    def chain_soa(self, inputs, dtype):
+        """Six arrays -> array of shape (7, n): w and the six gradients."""
+        dtype = np.dtype(dtype)
+        arrays = [np.ascontiguousarray(a, dtype=dtype) for a in inputs]
+        n = arrays[0].size
+        outs = [np.empty(n, dtype) for _ in range(7)]
+        fn = getattr(self.lib, "oracle_chain_soa" + _SUF[dtype])
+        fn.restype = None
+        fn(ctypes.c_long(n), *[a.ctypes.data_as(ctypes.c_void_p) for a in arrays],
+           *[a.ctypes.data_as(ctypes.c_void_p) for a in outs])
+        return np.stack(outs)
+
+    def set_threads(self, n):
+        self.lib.oracle_set_threads(ctypes.c_int(n))
+
+    def max_threads(self):
+        return self.lib.oracle_max_threads()

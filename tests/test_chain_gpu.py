@@ -1,0 +1,127 @@
+"""GPU parity of the per-thread forward+backward kernels, through the C ABI.
+
+Tolerances (fp32): the forward value within 1e-5 (abs-or-rel, the reference
+testers' measure) on every problem; gradients within 1e-5 wherever the
+covariance is well conditioned and within 1e-5 x cond(Sigma) in general, against
+both the fp32 and the fp64 oracle.  The fp32 oracle itself is only that close to
+fp64 (tests/test_oracle_chain.py), so nothing tighter is meaningful.
+"""
+import numpy as np
+import pytest
+
+from tests._metrics import abs_or_rel, chain_closed_form, chain_inputs, covariance_condition
+
+pytestmark = pytest.mark.gpu
+
+
+def _run_gpu(inputs, gpu, offset=0):
+    import torch
+
+    from xyz_autodiff_cuda_amd import chain
+
+    n = inputs[0].size
+    dev = []
+    for a in inputs:
+        buf = torch.empty(n + offset, dtype=torch.float32, device=gpu)
+        view = buf[offset:]
+        view.copy_(torch.from_numpy(np.ascontiguousarray(a)))
+        dev.append(view)
+    outs = [torch.full((n + offset,), float("nan"), dtype=torch.float32, device=gpu)[offset:] for _ in range(7)]
+    chain.forward_backward(dev, outs)
+    torch.cuda.synchronize()
+    return np.stack([o.cpu().numpy() for o in outs])
+
+
+def _check(got, inputs, oracle):
+    ref32 = oracle.chain_soa(inputs, np.float32)
+    ref64 = oracle.chain_soa(inputs, np.float64)
+    kappa = covariance_condition(inputs[0], inputs[1])
+    assert np.isfinite(got).all()
+    for ref in (ref32, ref64):
+        e = abs_or_rel(got, ref)
+        assert e[0].max() < 1e-5
+        assert e[:, kappa <= 7.4].max() < 1e-5
+        assert (e / np.maximum(1.0, kappa)).max() < 1e-5
+    assert abs_or_rel(got, ref64).max() <= 2.0 * abs_or_rel(ref32, ref64).max()
+
+
+@pytest.mark.parametrize("n", [1, 3, 4, 5, 255, 256, 257, 1023, 4096, 100003])
+def test_sizes_around_vector_and_block_edges(gpu, oracle, n):
+    inputs = chain_inputs(n, seed=100 + n)
+    _check(_run_gpu(inputs, gpu), inputs, oracle)
+
+
+def test_one_million_problems(gpu, oracle):
+    inputs = chain_inputs(1_000_000, seed=7)
+    got = _run_gpu(inputs, gpu)
+    _check(got, inputs, oracle)
+    # independent closed form, fp64
+    want, _ = chain_closed_form(inputs)
+    kappa = covariance_condition(inputs[0], inputs[1])
+    assert (abs_or_rel(got, want) / np.maximum(1.0, kappa)).max() < 1e-5
+
+
+def test_unaligned_buffers_take_the_scalar_kernel(gpu, oracle):
+    inputs = chain_inputs(5000, seed=9)
+    a = _run_gpu(inputs, gpu, offset=0)
+    b = _run_gpu(inputs, gpu, offset=1)  # 4-byte aligned only
+    assert np.array_equal(a, b)
+
+
+def test_device_matches_host_build_of_the_same_templates(gpu, xad):
+    from xyz_autodiff_cuda_amd import chain
+
+    inputs = chain_inputs(300000, seed=13)
+    got = _run_gpu(inputs, gpu)
+    host = np.stack(chain.host_forward_backward(inputs, np.float32))
+    kappa = covariance_condition(inputs[0], inputs[1])
+    e = abs_or_rel(got, host)
+    assert e[0].max() < 1e-5
+    assert (e / np.maximum(1.0, kappa)).max() < 1e-5
+
+
+def test_empty(gpu, xad):
+    import torch
+
+    from xyz_autodiff_cuda_amd import chain
+
+    z = [torch.empty(0, dtype=torch.float32, device=gpu) for _ in range(6)]
+    outs = chain.forward_backward(z)
+    assert all(o.numel() == 0 for o in outs)
+
+
+def test_rejects_null_and_host_tensors(gpu, xad):
+    import torch
+
+    from xyz_autodiff_cuda_amd import _lib, chain
+
+    with pytest.raises(TypeError):
+        chain.forward_backward([torch.zeros(4)] * 6)
+    lib = _lib.load()
+    status = lib.xad_chain_forward_backward_f32(4, *([None] * 13), None)
+    assert status != 0 and b"null" in lib.xad_last_error()
+
+
+def test_full_size_finite_differences_property(gpu, oracle):
+    """At the benchmark's full size (64 Mi problems) the oracle is too slow to
+    run on everything: check all outputs are finite, a strided sample against the
+    oracle, and the identity d w / d o = w (1 - sigmoid(o)) on every problem."""
+    import torch
+
+    from xyz_autodiff_cuda_amd import chain, rng
+
+    n = 64 * 1024 * 1024
+    ins = [torch.empty(n, dtype=torch.float32, device=gpu) for _ in range(6)]
+    rng.chain_inputs_(ins, seed=1234)
+    outs = chain.forward_backward(ins)
+    torch.cuda.synchronize()
+    for o in outs:
+        assert bool(torch.isfinite(o).all())
+    w, d_o = outs[0].double(), outs[4].double()
+    sig = torch.sigmoid(ins[3].double())
+    ident = (d_o - w * (1 - sig)).abs()
+    assert float(ident.max()) < 1e-6
+    idx = torch.arange(0, n, 997, device=gpu)
+    sample = [t[idx].cpu().numpy() for t in ins]
+    got = np.stack([o[idx].cpu().numpy() for o in outs])
+    _check(got, sample, oracle)

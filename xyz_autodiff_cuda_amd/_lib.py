@@ -1,0 +1,67 @@
+"""ctypes binding of libxad_hip.so (declared in include/xad_capi.h).
+
+The library is loaded from this directory only.  There is no fallback: if it
+has not been built, importing any compute entry point raises.
+"""
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libxad_hip.so")
+
+XAD_OK = 0
+
+
+class XadError(RuntimeError):
+    """A C-ABI call returned a non-zero status."""
+
+
+_lib = None
+
+_f32p = ctypes.POINTER(ctypes.c_float)
+_f64p = ctypes.POINTER(ctypes.c_double)
+_i32p = ctypes.POINTER(ctypes.c_int32)
+_u64p = ctypes.POINTER(ctypes.c_uint64)
+_sz = ctypes.c_size_t
+_u64 = ctypes.c_uint64
+_vp = ctypes.c_void_p
+_int = ctypes.c_int
+_flt = ctypes.c_float
+
+# name -> argument types; every function returns int unless listed in _RESTYPE.
+SIGNATURES = {
+    "xad_last_error": [],
+    "xad_abi_version": [],
+    "xad_chain_forward_backward_f32": [_sz] + [_vp] * 13 + [_vp],
+    "xad_host_chain_forward_backward_f32": [_sz] + [_vp] * 13 + [_int],
+    "xad_host_chain_forward_backward_f64": [_sz] + [_vp] * 13 + [_int],
+    "xad_rng_uniform_f32": [_vp, _sz, _u64, _u64, _flt, _flt, _vp],
+    "xad_rng_normal_f32": [_vp, _sz, _u64, _u64, _flt, _flt, _vp],
+    "xad_host_rng_bits": [_vp, _sz, _u64, _u64, _u64],
+    "xad_host_rng_uniform_f32": [_vp, _sz, _u64, _u64, _flt, _flt],
+}
+_RESTYPE = {"xad_last_error": ctypes.c_char_p}
+
+
+def load():
+    """Returns the loaded library, loading it on first use."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            "libxad_hip.so is not built (expected at %s); run `python -m xyz_autodiff_cuda_amd.build`" % LIB_PATH
+        )
+    lib = ctypes.CDLL(LIB_PATH)
+    for name, argtypes in SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.argtypes = argtypes
+        fn.restype = _RESTYPE.get(name, ctypes.c_int)
+    _lib = lib
+    return lib
+
+
+def check(status, what):
+    if status != XAD_OK:
+        msg = load().xad_last_error().decode("utf-8", "replace")
+        raise XadError("%s failed with status %d: %s" % (what, status, msg))

@@ -1,0 +1,162 @@
+// Per-thread forward+backward of the benchmark graph over structure-of-arrays
+// buffers: the GPU kernels, the host-core build of the same body, and their
+// C-ABI entry points.
+//
+// Memory traffic per problem is fixed by the interface: 6 floats in, 7 floats
+// out, 52 bytes, each touched once.  The kernels therefore
+//   - let every lane own four consecutive problems, so each of the 13 arrays is
+//     accessed with one 16-byte instruction per lane (1 KiB per wavefront),
+//   - mark all accesses non-temporal (nothing is reused),
+//   - keep the whole graph in VGPRs: no LDS, no scratch, no atomics.
+#include <algorithm>
+#include <thread>
+#include <vector>
+
+#include <xyz_autodiff/soa.cuh>
+
+#include "chain.cuh"
+#include "common.cuh"
+
+namespace {
+
+using xyz_autodiff::soa::Quad;
+
+struct ChainBuffers {
+    const float* in[6];  // sx, sy, theta, o, px, py
+    float* out[7];       // w, d_sx, d_sy, d_theta, d_o, d_px, d_py
+};
+
+constexpr unsigned kBlock = 256;
+
+// One lane, four consecutive problems, 16-byte accesses.  `groups` = n / 4.
+__global__ void __launch_bounds__(kBlock) chain_quad_kernel(ChainBuffers buf, std::size_t groups) {
+    using namespace xyz_autodiff::soa;
+    const std::size_t g = static_cast<std::size_t>(blockIdx.x) * kBlock + threadIdx.x;
+    if (g >= groups) return;
+
+    Quad<float> in[6];
+#pragma unroll
+    for (int a = 0; a < 6; ++a) in[a] = load4_stream(buf.in[a], g);
+
+    Quad<float> out[7];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const auto r = xad_chain::forward_backward<float>(in[0][k], in[1][k], in[2][k], in[3][k], in[4][k], in[5][k]);
+        out[0][k] = r.w;
+        out[1][k] = r.d_sx;
+        out[2][k] = r.d_sy;
+        out[3][k] = r.d_theta;
+        out[4][k] = r.d_o;
+        out[5][k] = r.d_px;
+        out[6][k] = r.d_py;
+    }
+#pragma unroll
+    for (int a = 0; a < 7; ++a) store4_stream(buf.out[a], g, out[a]);
+}
+
+// One lane, one problem, 4-byte accesses: unaligned buffers and the tail.
+__global__ void __launch_bounds__(kBlock) chain_single_kernel(ChainBuffers buf, std::size_t first, std::size_t n) {
+    const std::size_t i = first + static_cast<std::size_t>(blockIdx.x) * kBlock + threadIdx.x;
+    if (i >= n) return;
+    const auto r = xad_chain::forward_backward<float>(buf.in[0][i], buf.in[1][i], buf.in[2][i], buf.in[3][i],
+                                                      buf.in[4][i], buf.in[5][i]);
+    buf.out[0][i] = r.w;
+    buf.out[1][i] = r.d_sx;
+    buf.out[2][i] = r.d_sy;
+    buf.out[3][i] = r.d_theta;
+    buf.out[4][i] = r.d_o;
+    buf.out[5][i] = r.d_px;
+    buf.out[6][i] = r.d_py;
+}
+
+template <typename T>
+void host_chain_range(std::size_t begin, std::size_t end, const T* const* in, T* const* out) {
+    for (std::size_t i = begin; i < end; ++i) {
+        const auto r = xad_chain::forward_backward<T>(in[0][i], in[1][i], in[2][i], in[3][i], in[4][i], in[5][i]);
+        out[0][i] = r.w;
+        out[1][i] = r.d_sx;
+        out[2][i] = r.d_sy;
+        out[3][i] = r.d_theta;
+        out[4][i] = r.d_o;
+        out[5][i] = r.d_px;
+        out[6][i] = r.d_py;
+    }
+}
+
+template <typename T>
+int host_chain(std::size_t n, const T* const* in, T* const* out, int num_threads) {
+    for (int a = 0; a < 6; ++a) XAD_REQUIRE(n == 0 || in[a], "host chain: input array %d is null", a);
+    for (int a = 0; a < 7; ++a) XAD_REQUIRE(n == 0 || out[a], "host chain: output array %d is null", a);
+    unsigned threads = num_threads > 0 ? static_cast<unsigned>(num_threads) : std::thread::hardware_concurrency();
+    if (threads == 0) threads = 1;
+    threads = static_cast<unsigned>(std::min<std::size_t>(threads, std::max<std::size_t>(n / 1024, 1)));
+    if (threads == 1) {
+        host_chain_range<T>(0, n, in, out);
+        return XAD_OK;
+    }
+    std::vector<std::thread> pool;
+    pool.reserve(threads);
+    const std::size_t chunk = (n + threads - 1) / threads;
+    for (unsigned t = 0; t < threads; ++t) {
+        const std::size_t b = std::min(n, t * chunk), e = std::min(n, b + chunk);
+        pool.emplace_back(host_chain_range<T>, b, e, in, out);
+    }
+    for (auto& th : pool) th.join();
+    return XAD_OK;
+}
+
+}  // namespace
+
+extern "C" int xad_chain_forward_backward_f32(std::size_t n, const float* sx, const float* sy, const float* theta,
+                                              const float* o, const float* px, const float* py, float* w,
+                                              float* d_sx, float* d_sy, float* d_theta, float* d_o, float* d_px,
+                                              float* d_py, void* stream) {
+    ChainBuffers buf{{sx, sy, theta, o, px, py}, {w, d_sx, d_sy, d_theta, d_o, d_px, d_py}};
+    if (n == 0) return XAD_OK;
+    bool vector_ok = true;
+    for (int a = 0; a < 6; ++a) {
+        XAD_REQUIRE(buf.in[a], "xad_chain_forward_backward_f32: input array %d is null", a);
+        vector_ok = vector_ok && xad::aligned16(buf.in[a]);
+    }
+    for (int a = 0; a < 7; ++a) {
+        XAD_REQUIRE(buf.out[a], "xad_chain_forward_backward_f32: output array %d is null", a);
+        vector_ok = vector_ok && xad::aligned16(buf.out[a]);
+    }
+    XAD_REQUIRE(n / 4 <= 0x7fffffffull * kBlock, "xad_chain_forward_backward_f32: n = %zu exceeds the grid limit", n);
+
+    hipStream_t s = xad::as_stream(stream);
+    const std::size_t groups = vector_ok ? n / 4 : 0;
+    if (groups) {
+        hipLaunchKernelGGL(chain_quad_kernel, dim3(xad::blocks_for(groups, kBlock)), dim3(kBlock), 0, s, buf, groups);
+        XAD_HIP_TRY(hipGetLastError());
+    }
+    const std::size_t done = groups * 4;
+    if (done < n) {
+        XAD_REQUIRE((n - done + kBlock - 1) / kBlock <= 0x7fffffffull,
+                    "xad_chain_forward_backward_f32: n = %zu exceeds the grid limit of the 4-byte kernel", n);
+        hipLaunchKernelGGL(chain_single_kernel, dim3(xad::blocks_for(n - done, kBlock)), dim3(kBlock), 0, s, buf,
+                           done, n);
+        XAD_HIP_TRY(hipGetLastError());
+    }
+    return XAD_OK;
+}
+
+extern "C" int xad_host_chain_forward_backward_f32(std::size_t n, const float* sx, const float* sy,
+                                                   const float* theta, const float* o, const float* px,
+                                                   const float* py, float* w, float* d_sx, float* d_sy,
+                                                   float* d_theta, float* d_o, float* d_px, float* d_py,
+                                                   int num_threads) {
+    const float* in[6] = {sx, sy, theta, o, px, py};
+    float* out[7] = {w, d_sx, d_sy, d_theta, d_o, d_px, d_py};
+    return host_chain<float>(n, in, out, num_threads);
+}
+
+extern "C" int xad_host_chain_forward_backward_f64(std::size_t n, const double* sx, const double* sy,
+                                                   const double* theta, const double* o, const double* px,
+                                                   const double* py, double* w, double* d_sx, double* d_sy,
+                                                   double* d_theta, double* d_o, double* d_px, double* d_py,
+                                                   int num_threads) {
+    const double* in[6] = {sx, sy, theta, o, px, py};
+    double* out[7] = {w, d_sx, d_sy, d_theta, d_o, d_px, d_py};
+    return host_chain<double>(n, in, out, num_threads);
+}
