@@ -15,8 +15,17 @@
 // ScaleRotationToCovariance3ParamLogic :142-212, factories :215-238).  The
 // backward rules apply the chain rule in the same order as there: first to the
 // entries of M, then to (sx, sy, theta).
+//
+// sin(theta) and cos(theta) are needed by forward and by backward.  The logic
+// object remembers the pair together with the angle it belongs to; backward
+// reuses it when the angle is bit-for-bit the one forward saw (always, inside a
+// graph: the comparison is then resolved at compile time and the second
+// evaluation disappears) and evaluates afresh otherwise, e.g. after the
+// numerical backward has perturbed the angle.
 
+#include <bit>
 #include <cstddef>
+#include <cstdint>
 #include <type_traits>
 
 #include <xyz_autodiff/concept/core_logic.cuh>
@@ -28,6 +37,22 @@ namespace op {
 
 namespace detail_cov {
 
+template <typename T>
+struct AngleMemo {
+    using Bits = std::conditional_t<sizeof(T) == 4, std::uint32_t, std::uint64_t>;
+    T angle = T(0), sn = T(0), cs = T(1);
+    bool filled = false;
+
+    XAD_INLINE void evaluate(T theta) {
+        math::sincos(theta, sn, cs);
+        angle = theta;
+        filled = true;
+    }
+    XAD_INLINE void lookup(T theta) {
+        if (!(filled && std::bit_cast<Bits>(theta) == std::bit_cast<Bits>(angle))) evaluate(theta);
+    }
+};
+
 // M and the pull-back of a gradient on M to (sx, sy, theta); shared by the
 // stand-alone and the fused node.
 template <typename T>
@@ -35,8 +60,7 @@ struct RotatedScale {
     T sx, sy, cs, sn;
     T m00, m01, m10, m11;
 
-    XAD_INLINE RotatedScale(T sx_, T sy_, T theta) : sx(sx_), sy(sy_) {
-        math::sincos(theta, sn, cs);
+    XAD_INLINE RotatedScale(T sx_, T sy_, const AngleMemo<T>& trig) : sx(sx_), sy(sy_), cs(trig.cs), sn(trig.sn) {
         m00 = sx * cs;
         m01 = -sy * sn;
         m10 = sx * sn;
@@ -61,8 +85,11 @@ struct CovarianceMatrixGenerationLogic {
     using Output = Variable<Dim, T>;
     static constexpr std::size_t outputDim = Dim;
 
+    mutable detail_cov::AngleMemo<T> trig_;
+
     XAD_INLINE void forward(Output& out, const Input1& scale, const Input2& rotation) const {
-        const detail_cov::RotatedScale<T> m(scale[0], scale[1], rotation[0]);
+        trig_.evaluate(rotation[0]);
+        const detail_cov::RotatedScale<T> m(scale[0], scale[1], trig_);
         out[0] = m.m00;
         out[1] = m.m01;
         out[2] = m.m10;
@@ -70,7 +97,8 @@ struct CovarianceMatrixGenerationLogic {
     }
 
     XAD_INLINE void backward(const Output& out, Input1& scale, Input2& rotation) const {
-        const detail_cov::RotatedScale<T> m(scale[0], scale[1], rotation[0]);
+        trig_.lookup(rotation[0]);
+        const detail_cov::RotatedScale<T> m(scale[0], scale[1], trig_);
         m.pull_back(out.grad(0), out.grad(1), out.grad(2), out.grad(3), scale, rotation);
     }
 };
@@ -108,15 +136,19 @@ struct ScaleRotationToCovariance3ParamLogic {
     using Output = Variable<Dim, T>;
     static constexpr std::size_t outputDim = Dim;
 
+    mutable detail_cov::AngleMemo<T> trig_;
+
     XAD_INLINE void forward(Output& out, const Input1& scale, const Input2& rotation) const {
-        const detail_cov::RotatedScale<T> m(scale[0], scale[1], rotation[0]);
+        trig_.evaluate(rotation[0]);
+        const detail_cov::RotatedScale<T> m(scale[0], scale[1], trig_);
         out[0] = m.m00 * m.m00 + m.m01 * m.m01;
         out[1] = m.m00 * m.m10 + m.m01 * m.m11;
         out[2] = m.m10 * m.m10 + m.m11 * m.m11;
     }
 
     XAD_INLINE void backward(const Output& out, Input1& scale, Input2& rotation) const {
-        const detail_cov::RotatedScale<T> m(scale[0], scale[1], rotation[0]);
+        trig_.lookup(rotation[0]);
+        const detail_cov::RotatedScale<T> m(scale[0], scale[1], trig_);
         const T g00 = out.grad(0), g01 = out.grad(1), g11 = out.grad(2);
         m.pull_back(g00 * T(2) * m.m00 + g01 * m.m10,
                     g00 * T(2) * m.m01 + g01 * m.m11,

@@ -47,9 +47,8 @@ int xad_abi_version(void);
  *   w = sigmoid(o) * exp(-q / 2);   outputs: w and d w / d (sx, sy, theta, o, px, py)
  *
  * Six device input arrays and seven device output arrays of n floats each; no
- * two output arrays may overlap each other or an input.  Arrays aligned to 16
- * bytes are processed with 16-byte loads and stores (four problems per lane);
- * any other alignment is served by the 4-byte kernel.  n may be 0.
+ * two output arrays may overlap each other or an input.  Any 4-byte alignment
+ * is accepted.  n may be 0.
  * Stands in for the per-Gaussian graph that gaussian_splatting_kernel builds
  * and runs per (pixel, Gaussian)
  * (examples/mini-gaussian-splatting/gaussian_splatting_kernel.cu:73-111) and for
@@ -61,6 +60,18 @@ int xad_chain_forward_backward_f32(size_t n,
                                    float* w, float* d_sx, float* d_sy, float* d_theta,
                                    float* d_o, float* d_px, float* d_py,
                                    void* stream);
+
+/* Same computation with the lane-to-address mapping chosen by the caller:
+ * problems_per_lane = 1 (4-byte accesses, the default mapping of the entry point
+ * above) or 4 (16-byte accesses; needs all arrays 16-byte aligned, otherwise, and
+ * for the last n % 4 problems, the 4-byte kernel is used).  Results are identical;
+ * exists so both mappings can be measured.  No counterpart in the reference. */
+int xad_chain_forward_backward_f32_layout(size_t n,
+                                          const float* sx, const float* sy, const float* theta,
+                                          const float* o, const float* px, const float* py,
+                                          float* w, float* d_sx, float* d_sy, float* d_theta,
+                                          float* d_o, float* d_px, float* d_py,
+                                          int problems_per_lane, void* stream);
 
 /* The same graph from the same templates, compiled for the host and run on
  * `num_threads` host threads (<= 0: all hardware threads).  Host pointers.

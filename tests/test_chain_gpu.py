@@ -14,7 +14,7 @@ from tests._metrics import abs_or_rel, chain_closed_form, chain_inputs, covarian
 pytestmark = pytest.mark.gpu
 
 
-def _run_gpu(inputs, gpu, offset=0):
+def _run_gpu(inputs, gpu, offset=0, problems_per_lane=None):
     import torch
 
     from xyz_autodiff_cuda_amd import chain
@@ -27,7 +27,7 @@ def _run_gpu(inputs, gpu, offset=0):
         view.copy_(torch.from_numpy(np.ascontiguousarray(a)))
         dev.append(view)
     outs = [torch.full((n + offset,), float("nan"), dtype=torch.float32, device=gpu)[offset:] for _ in range(7)]
-    chain.forward_backward(dev, outs)
+    chain.forward_backward(dev, outs, problems_per_lane=problems_per_lane)
     torch.cuda.synchronize()
     return np.stack([o.cpu().numpy() for o in outs])
 
@@ -40,15 +40,16 @@ def _check(got, inputs, oracle):
     for ref in (ref32, ref64):
         e = abs_or_rel(got, ref)
         assert e[0].max() < 1e-5
-        assert e[:, kappa <= 7.4].max() < 1e-5
+        assert e[:, kappa <= 7.4].max(initial=0.0) < 1e-5
         assert (e / np.maximum(1.0, kappa)).max() < 1e-5
     assert abs_or_rel(got, ref64).max() <= 2.0 * abs_or_rel(ref32, ref64).max()
 
 
-@pytest.mark.parametrize("n", [1, 3, 4, 5, 255, 256, 257, 1023, 4096, 100003])
-def test_sizes_around_vector_and_block_edges(gpu, oracle, n):
+@pytest.mark.parametrize("lanes", [None, 1, 4])
+@pytest.mark.parametrize("n", [1, 3, 4, 5, 255, 256, 257, 1023, 1024, 1025, 4096, 100003])
+def test_sizes_around_vector_and_block_edges(gpu, oracle, n, lanes):
     inputs = chain_inputs(n, seed=100 + n)
-    _check(_run_gpu(inputs, gpu), inputs, oracle)
+    _check(_run_gpu(inputs, gpu, problems_per_lane=lanes), inputs, oracle)
 
 
 def test_one_million_problems(gpu, oracle):
@@ -61,11 +62,13 @@ def test_one_million_problems(gpu, oracle):
     assert (abs_or_rel(got, want) / np.maximum(1.0, kappa)).max() < 1e-5
 
 
-def test_unaligned_buffers_take_the_scalar_kernel(gpu, oracle):
-    inputs = chain_inputs(5000, seed=9)
-    a = _run_gpu(inputs, gpu, offset=0)
-    b = _run_gpu(inputs, gpu, offset=1)  # 4-byte aligned only
+def test_both_lane_mappings_and_unaligned_buffers_agree_bitwise(gpu, oracle):
+    inputs = chain_inputs(5003, seed=9)
+    a = _run_gpu(inputs, gpu, offset=0, problems_per_lane=1)
+    b = _run_gpu(inputs, gpu, offset=0, problems_per_lane=4)
+    c = _run_gpu(inputs, gpu, offset=1, problems_per_lane=4)  # 4-byte aligned only: falls to 4-byte accesses
     assert np.array_equal(a, b)
+    assert np.array_equal(a, c)
 
 
 def test_device_matches_host_build_of_the_same_templates(gpu, xad):

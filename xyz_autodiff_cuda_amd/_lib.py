@@ -33,6 +33,7 @@ SIGNATURES = {
     "xad_last_error": [],
     "xad_abi_version": [],
     "xad_chain_forward_backward_f32": [_sz] + [_vp] * 13 + [_vp],
+    "xad_chain_forward_backward_f32_layout": [_sz] + [_vp] * 13 + [_int, _vp],
     "xad_host_chain_forward_backward_f32": [_sz] + [_vp] * 13 + [_int],
     "xad_host_chain_forward_backward_f64": [_sz] + [_vp] * 13 + [_int],
     "xad_rng_uniform_f32": [_vp, _sz, _u64, _u64, _flt, _flt, _vp],

@@ -27,6 +27,10 @@ FLAGS = [
     "-fno-gpu-sanitize",
     "-march=x86-64-v3",
     "-munsafe-fp-atomics",
+    # x + 0 folds away (gradients start from zero); fp32 division is v_rcp_f32
+    # based (2.5 ulp) instead of the IEEE sequence
+    "-fno-signed-zeros",
+    "-fno-hip-fp32-correctly-rounded-divide-sqrt",
     # keep v_pk_*_f32 out of the generated code
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",

@@ -23,12 +23,14 @@ def _require_cuda_f32(t, name, n):
         raise ValueError("%s must be a contiguous float32 tensor of %d elements" % (name, n))
 
 
-def forward_backward(inputs, outputs=None, stream=None):
+def forward_backward(inputs, outputs=None, stream=None, problems_per_lane=None):
     """Runs the graph for every problem on the GPU.
 
     inputs:  six float32 CUDA tensors (sx, sy, theta, o, px, py) of equal length n.
     outputs: optional seven preallocated float32 CUDA tensors; allocated if None.
     stream:  torch.cuda.Stream to launch on (default: the current stream).
+    problems_per_lane: None for the library default, or 1 / 4 to pick the
+             lane-to-address mapping explicitly (4 = 16-byte accesses).
     Returns the seven output tensors (w, d_sx, d_sy, d_theta, d_o, d_px, d_py).
     """
     import torch
@@ -46,10 +48,12 @@ def forward_backward(inputs, outputs=None, stream=None):
     for t, name in zip(outputs, OUTPUT_NAMES):
         _require_cuda_f32(t, name, n)
     s = stream if stream is not None else torch.cuda.current_stream(inputs[0].device)
+    ptrs = [t.data_ptr() for t in inputs] + [t.data_ptr() for t in outputs]
     with torch.cuda.device(inputs[0].device):
-        status = lib.xad_chain_forward_backward_f32(
-            n, *[t.data_ptr() for t in inputs], *[t.data_ptr() for t in outputs], s.cuda_stream
-        )
+        if problems_per_lane is None:
+            status = lib.xad_chain_forward_backward_f32(n, *ptrs, s.cuda_stream)
+        else:
+            status = lib.xad_chain_forward_backward_f32_layout(n, *ptrs, int(problems_per_lane), s.cuda_stream)
     _lib.check(status, "xad_chain_forward_backward_f32")
     return outputs
 

@@ -1,4 +1,6 @@
 // Device and host fills from the counter-based generator.
+#include <algorithm>
+
 #include "common.cuh"
 #include "rng.cuh"
 
