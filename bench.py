@@ -69,6 +69,51 @@ def host_templates(host_inputs):
     return {"value": n / best, "unit": "evals/s", "threads": threads, "n": n, "GBps": 52.0 * n / best / 1e9}
 
 
+def accumulate_report(ins, seed, with_oracle):
+    """Config 3: 16 Mi threads add their six gradients into P Zipf(1.1)-distributed
+    slots.  Times the naive per-thread global atomics against the staged path and
+    checks both against the oracle's fp64 sums."""
+    import numpy as np
+    import torch
+
+    from xyz_autodiff_cuda_amd import accumulate
+
+    dev = ins[0].device
+    n = min(ins[0].numel(), 16 * 1024 * 1024)
+    sub = [t[:n] for t in ins]
+    host = [t.cpu().numpy() for t in sub] if with_oracle else None
+    out = {"n": n, "bytes_per_thread": accumulate.BYTES_PER_THREAD, "slots": {}}
+    for num_slots in (64, 4096, 262144):
+        slot = torch.empty(n, dtype=torch.int32, device=dev)
+        accumulate.zipf_(slot, seed, 10, num_slots, 1.1)
+        grads = torch.zeros(num_slots, 6, dtype=torch.float32, device=dev)
+        entry = {}
+        ref = None
+        if with_oracle:
+            from tests import _oracle
+
+            ref = _oracle.load().accumulate_chain(host, slot.cpu().numpy(), num_slots, chain_in_double=True)
+        for name, reps in (("auto", 10), ("wave_lds", 5), ("lds_f32", 5), ("global_atomics", 1)):
+            times = []
+            for _ in range(reps + (1 if reps > 1 else 0)):
+                grads.zero_()
+                a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                a.record()
+                accumulate.accumulate_chain_gradients(sub, slot, grads, name)
+                b.record()
+                torch.cuda.synchronize()
+                times.append(a.elapsed_time(b))
+            ms = sorted(times[1:] if reps > 1 else times)[len(times[1:] if reps > 1 else times) // 2]
+            item = {"ms": ms, "GBps": (accumulate.BYTES_PER_THREAD * n + 24.0 * num_slots) / ms / 1e6}
+            if ref is not None:
+                got = grads.cpu().numpy().astype(np.float64)
+                item["max_err_over_mass"] = float((np.abs(got - ref[0]) / (ref[1] + 1e-30))[ref[1] > 1e-3].max())
+            entry[name] = item
+        entry["speedup_vs_global_atomics"] = entry["global_atomics"]["ms"] / entry["auto"]["ms"]
+        out["slots"][str(num_slots)] = entry
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -160,6 +205,7 @@ def main():
         "outputs_finite": finite,
         "mapping_GBps": alt,
     }
+    record["accumulate"] = accumulate_report(ins, args.seed, with_oracle=not args.no_cpu)
     if not args.no_cpu:
         sample_n = min(n, 8 * 1024 * 1024)
         host_inputs = [t[:sample_n].cpu().numpy() for t in ins]

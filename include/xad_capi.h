@@ -91,6 +91,45 @@ int xad_host_chain_forward_backward_f64(size_t n,
                                         int num_threads);
 
 /* ---------------------------------------------------------------------------
+ * Parallel gradient accumulation.  Thread i evaluates the graph above on
+ * (sx[i], ..., py[i]) and adds its six gradients (d_sx, d_sy, d_theta, d_o, d_px,
+ * d_py) into row slot[i] of `grads`, a device array of num_slots x 6 floats,
+ * row-major, which the caller has initialised (the kernel only adds).  Entries
+ * of slot outside [0, num_slots) contribute nothing.  Floating-point sums are
+ * accumulated in an order that varies from run to run.
+ * `strategy` selects how the sums reach HBM:
+ *   GLOBAL_ATOMICS  one global atomic per thread per element: the pattern of
+ *                   VariableRef::add_grad (include/xyz_autodiff/variable.cuh:48-50;
+ *                   tests/test_parallel_gradient_accumulation.cu:25-49);
+ *   AUTO            WAVE_LDS_SHALLOW for num_slots <= 8, LDS otherwise (the measured optimum);
+ *   LDS             per-block table of partial sums in LDS, written out once per
+ *                   block (the reference's shared-memory pattern,
+ *                   tests/test_shared_memory_atomic.cu:29-64, made persistent).
+ *                   The table is fp64 (ds_add_f64) while num_slots x 6 doubles fit
+ *                   in 144 KiB of LDS, else fp32; beyond 6144 slots 4096 fp32 rows
+ *                   are claimed on first use and the rest falls through to HBM.
+ *                   LDS_F32 forces the fp32 table;
+ *   WAVE_LDS        DPP pre-reduction of equal slots inside each wavefront (groups
+ *                   of >= 4 lanes, up to eight groups per call), then as LDS;
+ *                   WAVE_LDS_SHALLOW: at most two groups;
+ *   *_LEAVES        the same kernels with the graph's leaves bound straight to
+ *                   the accumulator (drop-in leaf type), element by element.
+ */
+#define XAD_ACCUMULATE_GLOBAL_ATOMICS 0
+#define XAD_ACCUMULATE_LDS 1
+#define XAD_ACCUMULATE_WAVE_LDS 2
+#define XAD_ACCUMULATE_WAVE_LDS_SHALLOW 3
+#define XAD_ACCUMULATE_LDS_LEAVES 4
+#define XAD_ACCUMULATE_GLOBAL_LEAVES 5
+#define XAD_ACCUMULATE_LDS_F32 6
+#define XAD_ACCUMULATE_AUTO 7
+int xad_accumulate_chain_gradients_f32(int strategy, size_t n,
+                                       const float* sx, const float* sy, const float* theta,
+                                       const float* o, const float* px, const float* py,
+                                       const int* slot, float* grads, int num_slots,
+                                       void* stream);
+
+/* ---------------------------------------------------------------------------
  * Synthetic inputs: counter-based generator, element i of a fill is a pure
  * function of (seed, stream_id, i).  The reference seeds std::mt19937 on the
  * host and uploads (examples/mini-gaussian-splatting/gaussian_parameters.cu:27-66);
@@ -100,6 +139,11 @@ int xad_rng_uniform_f32(float* dst, size_t n, uint64_t seed, uint64_t stream_id,
                         float lo, float hi, void* stream);
 int xad_rng_normal_f32(float* dst, size_t n, uint64_t seed, uint64_t stream_id,
                        float mean, float stddev, void* stream);
+/* Zipf(exponent) over {0, .., num_slots-1}: P(k) ~ (k+1)^-exponent, by inverse
+ * CDF (table built on the host in fp64, binary search on the device with 53
+ * random bits).  Synchronous: allocates and frees a temporary device table. */
+int xad_rng_zipf_i32(int* dst, size_t n, uint64_t seed, uint64_t stream_id,
+                     int num_slots, double exponent, void* stream);
 /* Host: the raw 64 random bits of elements first .. first+n-1. */
 int xad_host_rng_bits(uint64_t* dst, size_t n, uint64_t seed, uint64_t stream_id, uint64_t first);
 int xad_host_rng_uniform_f32(float* dst, size_t n, uint64_t seed, uint64_t stream_id,

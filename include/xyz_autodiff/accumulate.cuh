@@ -1,0 +1,265 @@
+#pragma once
+// Gradient accumulation for parameters shared by many threads.
+//
+// When thousands of lanes add into the same few gradient slots, one global
+// atomic per lane per element (what VariableRef::add_grad does, and all that
+// xyz-autodiff-cuda offers: include/xyz_autodiff/variable.cuh:48-50, exercised
+// by tests/test_parallel_gradient_accumulation.cu:25-49) serialises at the L2
+// channel that owns the hot cache line.  BlockAccumulator stages the sums on
+// chip instead, in up to three levels:
+//
+//   1. wavefront   lanes of one wavefront that hit the same slot are summed
+//                  with DPP row operations (no memory traffic at all) and only
+//                  the group's first lane goes on;
+//   2. block       the partial sums are added into a table in LDS with native
+//                  LDS floating-point atomics;
+//   3. device      once per block the table is written out with one global
+//                  atomic per touched element.
+//
+// The table's element type is a template parameter and defaults to double even
+// for float gradients.  Measured on MI355X with 16 wavefronts per CU: a
+// ds_add_f32 wavefront instruction occupies the LDS pipeline for 192 cycles
+// whatever its addresses (3 cycles per lane), a ds_add_f64 for 8 cycles when
+// the 64 addresses are distinct, plus about 3 cycles per lane that shares an
+// address with another.  So partial sums are kept in fp64 (which also makes them
+// more accurate than the fp32 running sums of plain atomics), and level 1 exists
+// to take the lanes that share a slot out of the LDS instruction: summing a
+// group of m lanes costs about 60 VALU issue cycles once and saves about
+// 3 m Width LDS cycles, which pays from m = 4 on (MinGroup).
+//
+// The LDS table holds `capacity` slots of Width values, stored element-major
+// (all slots' element 0, then element 1, ...) so that the lanes of one
+// instruction, which all address the same element, spread over the banks.  If
+// all num_slots fit, slot s uses row s.  Otherwise rows are claimed on first use through a tag
+// array (hashed, one probe, no eviction): a slot that finds its row taken by
+// another slot falls through to a global atomic.  Under skewed access the hot
+// slots arrive first and most often, so they own the rows.
+//
+// Collective-call rules: construct(), add(), add_one() and flush() must be
+// reached by every lane of every wavefront of the block, in uniform control
+// flow (lanes with nothing to add pass a negative slot); the block size must
+// be a multiple of 64.
+//
+// SlotRef<N, T, Acc> is a drop-in leaf: a VariableRef whose add_grad goes
+// through an accumulator, so graphs and op logic stay unchanged.
+
+#include <cstddef>
+#include <cstdint>
+
+#include <xyz_autodiff/concept/variable.cuh>
+#include <xyz_autodiff/detail/atomic.cuh>
+#include <xyz_autodiff/detail/config.cuh>
+
+#if defined(__HIPCC__)
+
+namespace xyz_autodiff {
+namespace accumulate {
+
+enum class Strategy {
+    GlobalAtomics,  // level 3 only: one global atomic per lane per element
+    LdsAtomics,     // levels 2 + 3
+    WaveThenLds,    // levels 1 + 2 + 3
+};
+
+namespace wave {
+
+__device__ __forceinline__ unsigned lane_id() { return __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u)); }
+
+__device__ __forceinline__ std::uint64_t ballot(bool predicate) { return __builtin_amdgcn_ballot_w64(predicate); }
+
+template <int Ctrl>
+__device__ __forceinline__ float dpp_add(float v) {
+    const int moved = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), Ctrl, 0xF, 0xF, true);
+    return v + __builtin_bit_cast(float, moved);
+}
+
+__device__ __forceinline__ float read_lane(float v, int lane) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
+}
+
+// Sum of v over all 64 lanes, returned to every lane.  Four DPP steps reduce
+// each row of 16 (quad swaps, then the two mirrors), four scalar reads combine
+// the rows.
+__device__ __forceinline__ float sum(float v) {
+    v = dpp_add<0xB1>(v);   // quad_perm [1,0,3,2]
+    v = dpp_add<0x4E>(v);   // quad_perm [2,3,0,1]
+    v = dpp_add<0x141>(v);  // row_half_mirror
+    v = dpp_add<0x140>(v);  // row_mirror
+    return (read_lane(v, 0) + read_lane(v, 16)) + (read_lane(v, 32) + read_lane(v, 48));
+}
+
+}  // namespace wave
+
+template <typename T, int Width, Strategy S = Strategy::LdsAtomics, int PeelRounds = 8, int MinGroup = 4,
+          typename TableT = double>
+class BlockAccumulator {
+    static_assert(sizeof(T) == 4 || S != Strategy::WaveThenLds, "the wavefront level is implemented for 4-byte values");
+
+public:
+    using table_type = TableT;
+    static constexpr int kEmpty = -1;
+
+    // Bytes of LDS the block must provide for `capacity` rows.
+    __host__ __device__ static constexpr std::size_t lds_bytes(int capacity, bool tagged) {
+        if (S == Strategy::GlobalAtomics) return 0;
+        return static_cast<std::size_t>(capacity) * Width * sizeof(TableT) + (tagged ? static_cast<std::size_t>(capacity) * 4 : 0);
+    }
+
+    // `lds`: at least lds_bytes(capacity, num_slots > capacity) bytes, 16-byte aligned.
+    // `capacity` must be a power of two when num_slots > capacity (tagged mode).
+    // `global`: num_slots x Width values, row-major, already initialised.
+    // Clears the table; ends with a block barrier.
+    __device__ BlockAccumulator(void* lds, int capacity, T* global, int num_slots)
+        : table_(static_cast<TableT*>(lds)),
+          tags_(reinterpret_cast<int*>(static_cast<TableT*>(lds) + static_cast<std::size_t>(capacity) * Width)),
+          global_(global),
+          capacity_(capacity),
+          num_slots_(num_slots),
+          tagged_(num_slots > capacity),
+          shift_(32 - __builtin_ctz(static_cast<unsigned>(capacity))) {
+        clear();
+    }
+
+    // Adds g[0..Width) to slot `slot` (no-op for slot < 0).
+    __device__ __forceinline__ void add(int slot, const T (&g)[Width]) {
+        if constexpr (S == Strategy::GlobalAtomics) {
+            if (slot >= 0) {
+#pragma unroll
+                for (int k = 0; k < Width; ++k) detail::atomic_add(global_ + static_cast<std::size_t>(slot) * Width + k, g[k]);
+            }
+        } else {
+            if constexpr (S == Strategy::WaveThenLds) slot = peel(slot, g);
+            if (slot >= 0) deposit(slot, g);
+        }
+    }
+
+    // Adds one value to element `element` of slot `slot`.
+    __device__ __forceinline__ void add_one(int slot, int element, T value) {
+        if constexpr (S == Strategy::GlobalAtomics) {
+            if (slot >= 0) detail::atomic_add(global_ + static_cast<std::size_t>(slot) * Width + element, value);
+        } else {
+            if (slot < 0) return;
+            const int row = find_row(slot);
+            if (row >= 0)
+                detail::atomic_add(table_ + element * capacity_ + row, static_cast<TableT>(value));
+            else
+                detail::atomic_add(global_ + static_cast<std::size_t>(slot) * Width + element, value);
+        }
+    }
+
+    // Writes the table out (one global atomic per non-zero element) and clears
+    // it, so the object can take another round of add().
+    __device__ void flush() {
+        if constexpr (S == Strategy::GlobalAtomics) return;
+        __syncthreads();
+        // e runs over the global layout (slot-major) so the atomics of a
+        // wavefront touch consecutive addresses.
+        const int rows = tagged_ ? capacity_ : num_slots_;
+        for (int e = threadIdx.x; e < rows * Width; e += blockDim.x) {
+            const int row = e / Width, element = e % Width;
+            const int slot = tagged_ ? tags_[row] : row;
+            const T v = static_cast<T>(table_[element * capacity_ + row]);
+            if (slot != kEmpty && v != T(0)) detail::atomic_add(global_ + static_cast<std::size_t>(slot) * Width + element, v);
+        }
+        __syncthreads();
+        clear();
+    }
+
+private:
+    __device__ void clear() {
+        if constexpr (S == Strategy::GlobalAtomics) return;
+        for (int e = threadIdx.x; e < capacity_ * Width; e += blockDim.x) table_[e] = TableT(0);
+        if (tagged_)
+            for (int e = threadIdx.x; e < capacity_; e += blockDim.x) tags_[e] = kEmpty;
+        __syncthreads();
+    }
+
+    // Row of the LDS table that holds `slot`, or -1 if the slot has none.
+    __device__ __forceinline__ int find_row(int slot) {
+        if (!tagged_) return slot;
+        const int row = static_cast<int>((static_cast<unsigned>(slot) * 2654435761u) >> shift_);
+        int owner = tags_[row];
+        if (owner == kEmpty) {
+            const int seen = atomicCAS(tags_ + row, kEmpty, slot);
+            owner = seen == kEmpty ? slot : seen;
+        }
+        return owner == slot ? row : -1;
+    }
+
+    __device__ __forceinline__ void deposit(int slot, const T (&g)[Width]) {
+        const int row = find_row(slot);
+        if (row >= 0) {
+#pragma unroll
+            for (int k = 0; k < Width; ++k) detail::atomic_add(table_ + k * capacity_ + row, static_cast<TableT>(g[k]));
+        } else {
+#pragma unroll
+            for (int k = 0; k < Width; ++k) detail::atomic_add(global_ + static_cast<std::size_t>(slot) * Width + k, g[k]);
+        }
+    }
+
+    // Level 1.  Take the slot of the first lane that is still waiting and find
+    // every lane with the same slot.  If they are at least MinGroup, sum their
+    // values across the wavefront, let the first of them deposit the sums, and
+    // look at the next waiting lane (at most PeelRounds groups per call);
+    // otherwise stop: under skewed access a small leading group means the rest
+    // of the wavefront is scattered too, and those lanes are cheaper to deposit
+    // directly.  Returns the slot this lane still has to deposit itself (-1 if
+    // its contribution has been taken care of).
+    __device__ __forceinline__ int peel(int slot, const T (&g)[Width]) {
+        std::uint64_t waiting = wave::ballot(slot >= 0);
+        for (int round = 0; round < PeelRounds && waiting != 0; ++round) {
+            const int leader = __builtin_ctzll(waiting);
+            const int leader_slot = __builtin_amdgcn_readlane(slot, leader);
+            const bool member = slot == leader_slot;
+            const std::uint64_t group = wave::ballot(member);
+            if (__builtin_popcountll(group) < MinGroup) break;
+            waiting &= ~group;
+            T total[Width];
+#pragma unroll
+            for (int k = 0; k < Width; ++k) total[k] = wave::sum(member ? g[k] : T(0));
+            if (static_cast<int>(wave::lane_id()) == leader) deposit(leader_slot, total);
+            if (member) slot = -1;
+        }
+        return slot;
+    }
+
+    TableT* table_;
+    int* tags_;
+    T* global_;
+    int capacity_;
+    int num_slots_;
+    bool tagged_;
+    int shift_;
+};
+
+// A leaf that reads its values like a VariableRef and sends its gradients to a
+// BlockAccumulator: element i of this leaf is element `offset + i` of slot
+// `slot` in the accumulator's table.  zero_grad() is a no-op (the table is
+// owned and cleared by the accumulator); grad(i) is not readable before the
+// accumulator has been flushed, and returns the global value.
+template <std::size_t N, typename T, typename Acc>
+class SlotRef {
+public:
+    using value_type = T;
+    static constexpr std::size_t size = N;
+
+    __device__ SlotRef(T* values, Acc& acc, int slot, int offset, const T* global_grads)
+        : values_(values), acc_(&acc), grads_(global_grads), slot_(slot), offset_(offset) {}
+
+    __device__ __forceinline__ T& operator[](std::size_t i) const { return values_[i]; }
+    __device__ __forceinline__ const T& grad(std::size_t i) const { return grads_[i]; }
+    __device__ __forceinline__ void add_grad(std::size_t i, T g) const { acc_->add_one(slot_, offset_ + static_cast<int>(i), g); }
+    __device__ __forceinline__ void zero_grad() const {}
+
+private:
+    T* values_;
+    Acc* acc_;
+    const T* grads_;
+    int slot_;
+    int offset_;
+};
+
+}  // namespace accumulate
+}  // namespace xyz_autodiff
+
+#endif  // __HIPCC__

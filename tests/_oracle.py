@@ -77,3 +77,17 @@ class Oracle:
 
     def max_threads(self):
         return self.lib.oracle_max_threads()
+
+    def accumulate_chain(self, inputs, slot, num_slots, chain_in_double=True):
+        """fp64 per-slot sums of the six chain gradients and of their magnitudes: two (num_slots, 6) arrays."""
+        arrays = [np.ascontiguousarray(a, dtype=np.float32) for a in inputs]
+        slot = np.ascontiguousarray(slot, dtype=np.int32)
+        n = slot.size
+        sums = np.zeros((num_slots, 6), np.float64)
+        mass = np.zeros((num_slots, 6), np.float64)
+        fn = self.lib.oracle_accumulate_chain
+        fn.restype = None
+        fn(ctypes.c_long(n), *[a.ctypes.data_as(ctypes.c_void_p) for a in arrays], slot.ctypes.data_as(ctypes.c_void_p),
+           ctypes.c_int(num_slots), ctypes.c_int(1 if chain_in_double else 0),
+           sums.ctypes.data_as(ctypes.c_void_p), mass.ctypes.data_as(ctypes.c_void_p))
+        return sums, mass

@@ -36,6 +36,8 @@ SIGNATURES = {
     "xad_chain_forward_backward_f32_layout": [_sz] + [_vp] * 13 + [_int, _vp],
     "xad_host_chain_forward_backward_f32": [_sz] + [_vp] * 13 + [_int],
     "xad_host_chain_forward_backward_f64": [_sz] + [_vp] * 13 + [_int],
+    "xad_accumulate_chain_gradients_f32": [_int, _sz] + [_vp] * 8 + [_int, _vp],
+    "xad_rng_zipf_i32": [_vp, _sz, _u64, _u64, _int, ctypes.c_double, _vp],
     "xad_rng_uniform_f32": [_vp, _sz, _u64, _u64, _flt, _flt, _vp],
     "xad_rng_normal_f32": [_vp, _sz, _u64, _u64, _flt, _flt, _vp],
     "xad_host_rng_bits": [_vp, _sz, _u64, _u64, _u64],

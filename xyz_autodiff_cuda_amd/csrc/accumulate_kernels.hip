@@ -1,0 +1,243 @@
+// Parallel gradient accumulation: every thread evaluates the benchmark graph
+// for its own inputs and adds its six gradients into one of P shared slots.
+//
+// Three interchangeable strategies (see xyz_autodiff/accumulate.cuh): naive
+// global atomics, LDS table + one write-out per block, and wavefront
+// pre-reduction in front of the LDS table.  Blocks are persistent: the grid is
+// sized to the machine and each block walks a contiguous chunk of threads, so
+// the write-out of its table (the only global atomics of the staged
+// strategies) is amortised over as many threads as possible.
+#include <algorithm>
+#include <cmath>
+#include <vector>
+
+#include <xyz_autodiff/accumulate.cuh>
+
+#include "chain.cuh"
+#include "common.cuh"
+#include "rng.cuh"
+
+namespace {
+
+using xyz_autodiff::accumulate::BlockAccumulator;
+using xyz_autodiff::accumulate::Strategy;
+
+constexpr unsigned kBlock = 1024;
+constexpr int kWidth = 6;
+constexpr std::size_t kMaxLdsBytes = 160 * 1024;
+
+struct AccumulateArgs {
+    const float* in[6];  // sx, sy, theta, o, px, py
+    const int* slot;
+    float* grads;  // num_slots x 6
+    std::size_t n;
+    std::size_t per_block;  // multiple of kBlock
+    int num_slots;
+    int capacity;
+};
+
+template <Strategy S, int Peel, typename TableT>
+__global__ void __launch_bounds__(kBlock) accumulate_kernel(AccumulateArgs a) {
+    extern __shared__ __attribute__((aligned(16))) float lds[];
+    BlockAccumulator<float, kWidth, S, Peel, 4, TableT> acc(lds, a.capacity, a.grads, a.num_slots);
+
+    const std::size_t begin = static_cast<std::size_t>(blockIdx.x) * a.per_block;
+    const std::size_t end = begin + a.per_block < a.n ? begin + a.per_block : a.n;
+    for (std::size_t base = begin; base < end; base += kBlock) {
+        const std::size_t i = base + threadIdx.x;
+        int slot = -1;
+        float g[kWidth] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        if (i < end) {
+            float x[6];
+#pragma unroll
+            for (int k = 0; k < 6; ++k) x[k] = __builtin_nontemporal_load(a.in[k] + i);
+            const int s = __builtin_nontemporal_load(a.slot + i);
+            const auto r = xad_chain::forward_backward<float>(x[0], x[1], x[2], x[3], x[4], x[5]);
+            g[0] = r.d_sx;
+            g[1] = r.d_sy;
+            g[2] = r.d_theta;
+            g[3] = r.d_o;
+            g[4] = r.d_px;
+            g[5] = r.d_py;
+            // a slot outside [0, num_slots) is dropped rather than written out of bounds
+            slot = static_cast<unsigned>(s) < static_cast<unsigned>(a.num_slots) ? s : -1;
+        }
+        acc.add(slot, g);
+    }
+    acc.flush();
+}
+
+// Same work with the accumulator used through drop-in leaves: the graph is
+// written with SlotRef leaves in place of VariableRef leaves, and every
+// add_grad of the backward pass goes through the LDS table one element at a time.
+template <Strategy S, typename TableT>
+__global__ void __launch_bounds__(kBlock) accumulate_leaf_kernel(AccumulateArgs a) {
+    using namespace xyz_autodiff;
+    using Acc = BlockAccumulator<float, kWidth, S, 0, 4, TableT>;
+    extern __shared__ __attribute__((aligned(16))) float lds[];
+    Acc acc(lds, a.capacity, a.grads, a.num_slots);
+
+    const std::size_t begin = static_cast<std::size_t>(blockIdx.x) * a.per_block;
+    const std::size_t end = begin + a.per_block < a.n ? begin + a.per_block : a.n;
+    for (std::size_t base = begin; base < end; base += kBlock) {
+        const std::size_t i = base + threadIdx.x;
+        if (i < end) {
+            float x[6];
+#pragma unroll
+            for (int k = 0; k < 6; ++k) x[k] = __builtin_nontemporal_load(a.in[k] + i);
+            const int raw = __builtin_nontemporal_load(a.slot + i);
+            const int slot = static_cast<unsigned>(raw) < static_cast<unsigned>(a.num_slots) ? raw : -1;
+            const float* row = a.grads + static_cast<std::size_t>(slot < 0 ? 0 : slot) * kWidth;
+            accumulate::SlotRef<2, float, Acc> s(x + 0, acc, slot, 0, row + 0);
+            accumulate::SlotRef<1, float, Acc> theta(x + 2, acc, slot, 2, row + 2);
+            accumulate::SlotRef<1, float, Acc> opacity(x + 3, acc, slot, 3, row + 3);
+            accumulate::SlotRef<2, float, Acc> p(x + 4, acc, slot, 4, row + 4);
+            auto es = op::exp(s);
+            auto cov = op::scale_rotation_to_covariance_3param(es, theta);
+            auto inv = op::sym_matrix2_inv(cov);
+            auto q = op::mahalanobis_distance(p, inv);
+            auto half_q = q * 0.5f;
+            auto neg_half_q = op::neg(half_q);
+            auto falloff = op::exp(neg_half_q);
+            auto alpha = op::sigmoid(opacity);
+            auto w = falloff * alpha;
+            w.run();
+        }
+    }
+    acc.flush();
+}
+
+__global__ void __launch_bounds__(256) zipf_kernel(int* dst, std::size_t n, std::uint64_t key, const double* cdf,
+                                                   int num_slots) {
+    const std::size_t stride = static_cast<std::size_t>(gridDim.x) * 256;
+    for (std::size_t i = static_cast<std::size_t>(blockIdx.x) * 256 + threadIdx.x; i < n; i += stride) {
+        const double u = static_cast<double>(xad_rng::bits(key, i) >> 11) * 0x1.0p-53;
+        // first k with cdf[k] > u
+        int lo = 0, hi = num_slots - 1;
+        while (lo < hi) {
+            const int mid = (lo + hi) >> 1;
+            if (cdf[mid] > u)
+                hi = mid;
+            else
+                lo = mid + 1;
+        }
+        dst[i] = lo;
+    }
+}
+
+int device_compute_units(int* out) {
+    int dev = 0;
+    XAD_HIP_TRY(hipGetDevice(&dev));
+    hipDeviceProp_t prop;
+    XAD_HIP_TRY(hipGetDeviceProperties(&prop, dev));
+    *out = prop.multiProcessorCount;
+    return XAD_OK;
+}
+
+template <typename Kernel>
+int launch(Kernel kernel, AccumulateArgs a, std::size_t lds_bytes, int blocks_per_cu, void* stream) {
+    int cus = 0;
+    if (int st = device_compute_units(&cus)) return st;
+    if (lds_bytes > 64 * 1024)
+        XAD_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                        static_cast<int>(lds_bytes)));
+    const std::size_t chunks = (a.n + kBlock - 1) / kBlock;
+    std::size_t blocks = std::min<std::size_t>(chunks, static_cast<std::size_t>(cus) * blocks_per_cu);
+    const std::size_t chunks_per_block = (chunks + blocks - 1) / blocks;
+    a.per_block = chunks_per_block * kBlock;
+    blocks = (a.n + a.per_block - 1) / a.per_block;
+    hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(blocks)), dim3(kBlock), lds_bytes, xad::as_stream(stream), a);
+    XAD_HIP_TRY(hipGetLastError());
+    return XAD_OK;
+}
+
+}  // namespace
+
+extern "C" int xad_accumulate_chain_gradients_f32(int strategy, std::size_t n, const float* sx, const float* sy,
+                                                  const float* theta, const float* o, const float* px,
+                                                  const float* py, const int* slot, float* grads, int num_slots,
+                                                  void* stream) {
+    const char* who = "xad_accumulate_chain_gradients_f32";
+    if (n == 0) return XAD_OK;
+    AccumulateArgs a{{sx, sy, theta, o, px, py}, slot, grads, n, 0, num_slots, 0};
+    for (int k = 0; k < 6; ++k) XAD_REQUIRE(a.in[k], "%s: input array %d is null", who, k);
+    XAD_REQUIRE(slot && grads, "%s: slot or grads is null", who);
+    XAD_REQUIRE(num_slots > 0, "%s: num_slots must be positive, got %d", who, num_slots);
+
+    // Strategy AUTO: wavefront pre-reduction only pays when nearly all lanes of a
+    // wavefront share a slot (measured: a win up to about 8 slots).
+    if (strategy == XAD_ACCUMULATE_AUTO) strategy = num_slots <= 8 ? XAD_ACCUMULATE_WAVE_LDS_SHALLOW : XAD_ACCUMULATE_LDS;
+
+    // LDS table (at most 144 KiB): fp64 rows for every slot if they fit; otherwise fp32
+    // rows for every slot if those fit (the slower ds_add_f32 still beats sending the
+    // overflow to HBM); otherwise 4096 fp32 rows claimed on first use.
+    constexpr std::size_t kTableBudget = 144 * 1024;
+    const std::size_t cells = static_cast<std::size_t>(num_slots) * kWidth;
+    bool f32_table = strategy == XAD_ACCUMULATE_LDS_F32;
+    if (!f32_table && cells * sizeof(double) > kTableBudget) f32_table = true;
+    const std::size_t cell = f32_table ? sizeof(float) : sizeof(double);
+    const bool direct = cells * cell <= kTableBudget;
+    a.capacity = direct ? num_slots : 4096;
+    const std::size_t lds = static_cast<std::size_t>(a.capacity) * kWidth * cell + (direct ? 0 : a.capacity * 4u);
+    XAD_REQUIRE(lds <= kMaxLdsBytes, "%s: LDS table of %zu bytes does not fit", who, lds);
+    const int per_cu = lds <= 32 * 1024 ? 2 : 1;
+    if (f32_table && strategy != XAD_ACCUMULATE_GLOBAL_ATOMICS && strategy != XAD_ACCUMULATE_GLOBAL_LEAVES) {
+        switch (strategy) {
+            case XAD_ACCUMULATE_WAVE_LDS:
+                return launch(accumulate_kernel<Strategy::WaveThenLds, 8, float>, a, lds, per_cu, stream);
+            case XAD_ACCUMULATE_WAVE_LDS_SHALLOW:
+                return launch(accumulate_kernel<Strategy::WaveThenLds, 2, float>, a, lds, per_cu, stream);
+            case XAD_ACCUMULATE_LDS_LEAVES:
+                return launch(accumulate_leaf_kernel<Strategy::LdsAtomics, float>, a, lds, per_cu, stream);
+            default:
+                return launch(accumulate_kernel<Strategy::LdsAtomics, 0, float>, a, lds, per_cu, stream);
+        }
+    }
+
+    switch (strategy) {
+        case XAD_ACCUMULATE_GLOBAL_ATOMICS:
+            return launch(accumulate_kernel<Strategy::GlobalAtomics, 0, double>, a, 0, 2, stream);
+        case XAD_ACCUMULATE_LDS:
+            return launch(accumulate_kernel<Strategy::LdsAtomics, 0, double>, a, lds, per_cu, stream);
+        case XAD_ACCUMULATE_WAVE_LDS:
+            return launch(accumulate_kernel<Strategy::WaveThenLds, 8, double>, a, lds, per_cu, stream);
+        case XAD_ACCUMULATE_WAVE_LDS_SHALLOW:
+            return launch(accumulate_kernel<Strategy::WaveThenLds, 2, double>, a, lds, per_cu, stream);
+        case XAD_ACCUMULATE_LDS_LEAVES:
+            return launch(accumulate_leaf_kernel<Strategy::LdsAtomics, double>, a, lds, per_cu, stream);
+        case XAD_ACCUMULATE_GLOBAL_LEAVES:
+            return launch(accumulate_leaf_kernel<Strategy::GlobalAtomics, double>, a, 0, 2, stream);
+        default:
+            return xad::fail(XAD_ERR_INVALID_ARGUMENT, "%s: unknown strategy %d", who, strategy);
+    }
+}
+
+extern "C" int xad_rng_zipf_i32(int* dst, std::size_t n, std::uint64_t seed, std::uint64_t stream_id, int num_slots,
+                                double exponent, void* stream) {
+    const char* who = "xad_rng_zipf_i32";
+    if (n == 0) return XAD_OK;
+    XAD_REQUIRE(dst, "%s: destination is null", who);
+    XAD_REQUIRE(num_slots > 0 && exponent > 0.0, "%s: need num_slots > 0 and exponent > 0", who);
+    std::vector<double> cdf(static_cast<std::size_t>(num_slots));
+    double total = 0.0;
+    for (int k = 0; k < num_slots; ++k) total += std::pow(static_cast<double>(k + 1), -exponent);
+    double running = 0.0;
+    for (int k = 0; k < num_slots; ++k) {
+        running += std::pow(static_cast<double>(k + 1), -exponent);
+        cdf[k] = running / total;
+    }
+    cdf[num_slots - 1] = 2.0;  // the search never runs off the end
+    double* d_cdf = nullptr;
+    XAD_HIP_TRY(hipMalloc(&d_cdf, cdf.size() * sizeof(double)));
+    hipError_t st = hipMemcpy(d_cdf, cdf.data(), cdf.size() * sizeof(double), hipMemcpyHostToDevice);
+    if (st == hipSuccess) {
+        const unsigned grid = static_cast<unsigned>(std::min<std::size_t>((n + 255) / 256, 256u * 32u));
+        hipLaunchKernelGGL(zipf_kernel, dim3(grid), dim3(256), 0, xad::as_stream(stream), dst, n,
+                           xad_rng::stream_key(seed, stream_id), d_cdf, num_slots);
+        st = hipGetLastError();
+        if (st == hipSuccess) st = hipStreamSynchronize(xad::as_stream(stream));
+    }
+    (void)hipFree(d_cdf);
+    if (st != hipSuccess) return xad::fail(XAD_ERR_HIP, "%s: %s", who, hipGetErrorString(st));
+    return XAD_OK;
+}
