@@ -130,6 +130,63 @@ int xad_accumulate_chain_gradients_f32(int strategy, size_t n,
                                        void* stream);
 
 /* ---------------------------------------------------------------------------
+ * Tile-binned 2D Gaussian splatting: render, loss and parameter gradients.
+ *
+ * Stands in for launch_gaussian_splatting of the reference example
+ * (examples/mini-gaussian-splatting/gaussian_splatting_kernel.cu:114-149), which
+ * renders, accumulates the loss and accumulates all gradients in one launch, and
+ * for zero_gradients_gpu (gaussian_parameters.cu:243-257): gradients are written,
+ * not added, so no separate zeroing call exists.  The per-Gaussian opacity graph
+ * is the reference's; the renderer around it is the one the benchmark
+ * configuration specifies (16x16 tiles, 3-sigma box binning, (depth, index)
+ * order, front-to-back compositing with alpha <= 0.99, stop below T = 1e-4, sum
+ * of squared errors), not the reference's additive all-pairs renderer.
+ *
+ *   params  device, 9 rows of G floats: cx, cy, log-scale x, log-scale y, theta,
+ *           r, g, b, opacity logit (the fields of GaussianParams,
+ *           gaussian_parameters.h:12-18, as a structure of arrays)
+ *   depth   device, G floats (ordering only; not differentiated)
+ *   target, image   device, height x width x 3 floats, interleaved RGB
+ *   grads   device, 9 rows of G floats, overwritten
+ *
+ * The context owns all intermediate device buffers (records, pair lists, sort
+ * workspace, per-pixel state); they grow when a step produces more (tile,
+ * Gaussian) pairs than fit.  A step reads one 4-byte count back to size the
+ * sort, so calls synchronise with `stream` once.  One context serves one stream
+ * at a time.
+ */
+typedef struct xad_splat_context xad_splat_context;
+int xad_splat_create(int width, int height, int num_gaussians, size_t pair_capacity_hint,
+                     xad_splat_context** out);
+void xad_splat_destroy(xad_splat_context* ctx);
+/* Render only. */
+int xad_splat_forward(xad_splat_context* ctx, const float* params, const float* depth,
+                      float* image, void* stream);
+/* Render, loss and gradients.  loss_out (host, may be NULL) receives the sum of
+ * squared errors; passing it makes the call wait for the stream. */
+int xad_splat_step(xad_splat_context* ctx, const float* params, const float* depth,
+                   const float* target, float* image, float* grads, double* loss_out,
+                   void* stream);
+/* Per-stage GPU times (events around project, scan+emit, sort, tile ranges,
+ * render forward, render backward, parameter backward) are recorded by the next
+ * calls when enabled; recording makes each call wait for the stream. */
+int xad_splat_set_profiling(xad_splat_context* ctx, int enabled);
+/* Of the last call: number of (tile, Gaussian) pairs, longest tile list, and the
+ * seven stage times in milliseconds (zeros unless profiling is enabled).  Any
+ * output pointer may be NULL. */
+int xad_splat_get_stats(const xad_splat_context* ctx, uint64_t* pairs, uint32_t* longest_list,
+                        float* stage_ms);
+
+/* Adam over structure-of-arrays parameters: `rows` rows of n floats each in
+ * params, grads, m and v (device); row r uses row_learning_rates[r] (host).
+ * iteration counts from 1.  Arithmetic of adam_step_individual_kernel
+ * (examples/mini-gaussian-splatting/gaussian_parameters.cu:260-320, launcher
+ * :353-386); no clamping. */
+int xad_adam_step_f32(size_t n, int rows, float* params, const float* grads, float* m, float* v,
+                      const float* row_learning_rates, float beta1, float beta2, float eps,
+                      int iteration, void* stream);
+
+/* ---------------------------------------------------------------------------
  * Synthetic inputs: counter-based generator, element i of a fill is a pure
  * function of (seed, stream_id, i).  The reference seeds std::mt19937 on the
  * host and uploads (examples/mini-gaussian-splatting/gaussian_parameters.cu:27-66);

@@ -91,3 +91,48 @@ class Oracle:
            ctypes.c_int(num_slots), ctypes.c_int(1 if chain_in_double else 0),
            sums.ctypes.data_as(ctypes.c_void_p), mass.ctypes.data_as(ctypes.c_void_p))
         return sums, mass
+
+    # ---- splatting -----------------------------------------------------------
+
+    def splat_step(self, width, height, params, depth, target, dtype=np.float32, want_grads=True):
+        """Tile-binned step on the CPU.  params (9, G).  Returns dict with image (H, W, 3),
+        grads (9, G) or None, loss, pairs, longest_list, seconds (5 stages)."""
+        dtype = np.dtype(dtype)
+        params = np.ascontiguousarray(params, dtype=dtype)
+        depth = np.ascontiguousarray(depth, dtype=dtype)
+        target = np.ascontiguousarray(target, dtype=dtype)
+        G = params.shape[1]
+        image = np.zeros((height, width, 3), dtype)
+        grads = np.zeros((9, G), dtype) if want_grads else None
+        stats = (ctypes.c_long * 2)()
+        seconds = (ctypes.c_double * 5)()
+        fn = getattr(self.lib, "oracle_splat_step" + _SUF[dtype])
+        fn.restype = ctypes.c_double
+        P = ctypes.c_void_p
+        loss = fn(ctypes.c_int(width), ctypes.c_int(height), ctypes.c_int(G), params.ctypes.data_as(P), depth.ctypes.data_as(P),
+                  target.ctypes.data_as(P), image.ctypes.data_as(P), grads.ctypes.data_as(P) if want_grads else P(0), stats, seconds)
+        return {"image": image, "grads": grads, "loss": loss, "pairs": stats[0], "longest_list": stats[1], "seconds": list(seconds)}
+
+    def splat_bruteforce(self, width, height, params, depth, target, dtype=np.float64):
+        """Every pixel against every Gaussian.  Returns (image, loss)."""
+        dtype = np.dtype(dtype)
+        params = np.ascontiguousarray(params, dtype=dtype)
+        depth = np.ascontiguousarray(depth, dtype=dtype)
+        target = np.ascontiguousarray(target, dtype=dtype)
+        image = np.zeros((height, width, 3), dtype)
+        fn = getattr(self.lib, "oracle_splat_bruteforce" + _SUF[dtype])
+        fn.restype = ctypes.c_double
+        P = ctypes.c_void_p
+        loss = fn(ctypes.c_int(width), ctypes.c_int(height), ctypes.c_int(params.shape[1]), params.ctypes.data_as(P),
+                  depth.ctypes.data_as(P), target.ctypes.data_as(P), image.ctypes.data_as(P))
+        return image, loss
+
+    def adam_step(self, p, g, m, v, lr, beta1, beta2, eps, iteration):
+        """In place on float32 numpy arrays (any shape, one learning rate)."""
+        for a in (p, g, m, v):
+            assert a.dtype == np.float32 and a.flags["C_CONTIGUOUS"]
+        fn = self.lib.oracle_adam_step_f32
+        fn.restype = None
+        P = ctypes.c_void_p
+        fn(ctypes.c_long(p.size), p.ctypes.data_as(P), g.ctypes.data_as(P), m.ctypes.data_as(P), v.ctypes.data_as(P),
+           ctypes.c_float(lr), ctypes.c_float(beta1), ctypes.c_float(beta2), ctypes.c_float(eps), ctypes.c_int(iteration))

@@ -1,0 +1,168 @@
+"""Pins the splatting oracle.
+
+The reference has no tile-binned compositing renderer, so nothing in its tests
+pins these rules ("parity unpinned" by the reference); they are pinned by the
+mathematics instead: closed forms for one and two Gaussians, the alpha clamp and
+the transmittance cut-off, agreement of the tiled renderer with a brute-force
+O(W H G) renderer, invariance to the order in which Gaussians are listed, and
+central finite differences of the loss for every parameter.  The per-Gaussian
+part (exp, covariance, inverse, sigmoid, Mahalanobis) is the reference's op
+logic, pinned in tests/test_oracle_ops.py and tests/test_oracle_chain.py.
+"""
+import numpy as np
+import pytest
+
+from tests._scenes import one_gaussian, random_scene
+
+
+def sigmoid(x):
+    return 1.0 / (1.0 + np.exp(-x))
+
+
+def test_one_gaussian_closed_form(oracle):
+    W = H = 32
+    rgb = (0.2, 0.5, 0.9)
+    params = one_gaussian(10.0, 12.0, np.log(3.0), np.log(3.0), 0.0, rgb, 0.4)
+    depth = np.array([0.5], np.float32)
+    target = np.zeros((H, W, 3), np.float32)
+    out = oracle.splat_step(W, H, params, depth, target, np.float64)
+    a0 = sigmoid(np.float64(np.float32(0.4)))
+    # at the centre q = 0: C = alpha * colour
+    assert np.allclose(out["image"][12, 10], a0 * np.array(rgb, np.float32).astype(np.float64), rtol=1e-12)
+    # isotropic: alpha(r) = a0 exp(-r^2 / (2 s^2)) with s = exp(log 3)
+    s2 = np.exp(np.float64(np.float32(np.log(3.0)))) ** 2
+    for (x, y) in ((13, 12), (10, 17), (4, 9)):
+        r2 = (x - 10.0) ** 2 + (y - 12.0) ** 2
+        want = a0 * np.exp(-0.5 * r2 / s2) * np.float64(np.float32(rgb[0]))
+        assert np.isclose(out["image"][y, x, 0], want, rtol=1e-9)
+
+
+def test_two_gaussians_compose_front_to_back_by_depth(oracle):
+    W = H = 16
+    a = one_gaussian(8, 8, np.log(4.0), np.log(4.0), 0.0, (1, 0, 0), 0.0)
+    b = one_gaussian(8, 8, np.log(4.0), np.log(4.0), 0.0, (0, 1, 0), 1.0)
+    params = np.concatenate([a, b], axis=1)
+    target = np.zeros((H, W, 3), np.float32)
+    a1, a2 = sigmoid(0.0), sigmoid(1.0)
+    front_a = oracle.splat_step(W, H, params, np.array([0.1, 0.9], np.float32), target, np.float64)["image"][8, 8]
+    front_b = oracle.splat_step(W, H, params, np.array([0.9, 0.1], np.float32), target, np.float64)["image"][8, 8]
+    assert np.allclose(front_a, [a1, (1 - a1) * a2, 0.0], rtol=1e-12)
+    assert np.allclose(front_b, [(1 - a2) * a1, a2, 0.0], rtol=1e-12)
+    # equal depth: lower index in front
+    tie = oracle.splat_step(W, H, params, np.array([0.5, 0.5], np.float32), target, np.float64)["image"][8, 8]
+    assert np.allclose(tie, front_a, rtol=1e-12)
+
+
+def test_alpha_is_clamped_and_clamped_alpha_passes_no_gradient(oracle):
+    W = H = 16
+    params = one_gaussian(8, 8, np.log(1000.0), np.log(1000.0), 0.0, (1, 1, 1), 12.0)  # alpha > 0.99 everywhere in view
+    target = np.zeros((H, W, 3), np.float32)
+    out = oracle.splat_step(W, H, params, np.array([0.5], np.float32), target, np.float64)
+    assert np.allclose(out["image"], 0.99)
+    g = out["grads"][:, 0]
+    assert np.all(g[[0, 1, 2, 3, 4, 8]] == 0.0)  # nothing through alpha
+    assert np.allclose(g[5:8], 2 * 0.99 * 0.99 * W * H, rtol=1e-12)  # colour: sum 2 (C - 0) alpha T
+
+
+def test_transmittance_cutoff_stops_compositing(oracle):
+    W = H = 16
+    layers = [one_gaussian(8, 8, np.log(1000.0), np.log(1000.0), 0.0, (1.0, 0.0, 0.0), 12.0) for _ in range(5)]
+    layers[3][5:8, 0] = (0.0, 1.0, 0.0)  # the 4th layer is green: must never show
+    layers[4][5:8, 0] = (0.0, 0.0, 1.0)
+    params = np.concatenate(layers, axis=1)
+    depth = np.linspace(0.1, 0.9, 5).astype(np.float32)
+    target = np.zeros((H, W, 3), np.float32)
+    out = oracle.splat_step(W, H, params, depth, target, np.float64)
+    # T: 1 -> 0.01 -> 1e-4 (not below the threshold) -> 1e-6 -> stop: three layers drawn
+    want_red = 0.99 * (1 + 0.01 + 0.01 * 0.01)
+    assert np.allclose(out["image"][..., 0], want_red, rtol=1e-12)
+    assert np.all(out["image"][..., 1:] == 0.0)
+    assert np.all(out["grads"][:, 3:] == 0.0)
+
+
+@pytest.mark.parametrize("seed,G,W,H", [(1, 8, 32, 32), (2, 40, 48, 40), (3, 25, 33, 17)])
+def test_tiled_renderer_equals_brute_force(oracle, seed, G, W, H):
+    params, depth = random_scene(G, W, H, seed, scale_px=(1.0, 12.0))
+    target = np.random.default_rng(seed).uniform(0, 1, (H, W, 3)).astype(np.float32)
+    for dtype in (np.float64, np.float32):
+        tiled = oracle.splat_step(W, H, params, depth, target, dtype, want_grads=False)
+        image, loss = oracle.splat_bruteforce(W, H, params, depth, target, dtype)
+        assert np.array_equal(tiled["image"], image)  # same operations in the same order
+        assert np.isclose(tiled["loss"], loss, rtol=1e-12)
+
+
+def test_listing_order_of_gaussians_does_not_matter(oracle):
+    W, H, G = 40, 40, 30
+    params, depth = random_scene(G, W, H, 7, scale_px=(1.0, 10.0))
+    target = np.random.default_rng(7).uniform(0, 1, (H, W, 3)).astype(np.float32)
+    base = oracle.splat_step(W, H, params, depth, target, np.float64)
+    perm = np.random.default_rng(8).permutation(G)
+    shuffled = oracle.splat_step(W, H, params[:, perm], depth[perm], target, np.float64)
+    assert np.array_equal(base["image"], shuffled["image"])
+    assert np.allclose(base["grads"][:, perm], shuffled["grads"], rtol=1e-12, atol=1e-15)
+
+
+def test_gradients_match_central_differences_of_the_brute_force_loss(oracle):
+    W, H, G = 40, 32, 12
+    params, depth = random_scene(G, W, H, 11, scale_px=(2.0, 8.0))
+    target = np.random.default_rng(11).uniform(0, 1, (H, W, 3)).astype(np.float32)
+    p64 = params.astype(np.float64)
+    out = oracle.splat_step(W, H, p64, depth, target, np.float64)
+    h = 1e-6
+    worst = 0.0
+    for g in range(G):
+        for row in range(9):
+            hi, lo = p64.copy(), p64.copy()
+            hi[row, g] += h
+            lo[row, g] -= h
+            fd = (oracle.splat_bruteforce(W, H, hi, depth, target)[1] - oracle.splat_bruteforce(W, H, lo, depth, target)[1]) / (2 * h)
+            an = out["grads"][row, g]
+            err = min(abs(an - fd), abs(an - fd) / (abs(fd) + 1e-15))
+            worst = max(worst, err)
+            assert err < 1e-5, (g, row, an, fd)
+    assert worst < 1e-5
+
+
+def test_offscreen_and_nonfinite_gaussians_are_dropped(oracle):
+    W = H = 32
+    params, depth = random_scene(6, W, H, 5, scale_px=(1.0, 4.0))
+    params[0, 0] = -500.0  # far left of the image
+    params[1, 1] = 1e6
+    params[2, 2] = np.nan
+    target = np.zeros((H, W, 3), np.float32)
+    out = oracle.splat_step(W, H, params, depth, target, np.float32)
+    assert np.isfinite(out["image"]).all()
+    assert np.all(out["grads"][:, :2] == 0.0)  # off-screen: no pixel, no gradient
+    keep = oracle.splat_step(W, H, params[:, 3:], depth[3:], target, np.float32)
+    assert np.array_equal(out["image"], keep["image"])
+    assert np.array_equal(out["grads"][:, 3:], keep["grads"])  # a non-finite neighbour changes nothing for the others
+
+
+def test_adam_first_step_closed_form(oracle):
+    """From zero moments, step 1: m = (1-b1) g, v = (1-b2) g^2, so
+    p - p0 = -lr g / (|g| + eps / sqrt(1-b2)), i.e. about -lr sign(g)."""
+    r = np.random.default_rng(0)
+    g = r.normal(0, 3, 1000).astype(np.float32)
+    g[::50] = 0.0
+    p0 = r.normal(0, 1, 1000).astype(np.float32)
+    p, m, v = p0.copy(), np.zeros_like(p0), np.zeros_like(p0)
+    lr, b1, b2, eps = 1e-2, 0.9, 0.999, 1e-8
+    oracle.adam_step(p, g, m, v, lr, b1, b2, eps, 1)
+    want = p0.astype(np.float64) - lr * g / (np.abs(g.astype(np.float64)) + eps / np.sqrt(1 - b2))
+    assert np.allclose(p, want, rtol=2e-5, atol=1e-7)
+    assert np.allclose(m, (1 - b1) * g, rtol=1e-6) and np.allclose(v, (1 - b2) * g.astype(np.float64) ** 2, rtol=1e-4)  # 1 - 0.999f is 0.00100005 in fp32
+
+
+def test_adam_many_steps_match_fp64_recurrence(oracle):
+    r = np.random.default_rng(1)
+    p0 = r.normal(0, 1, 500).astype(np.float32)
+    p, m, v = p0.copy(), np.zeros_like(p0), np.zeros_like(p0)
+    pd, md, vd = p0.astype(np.float64), np.zeros(500), np.zeros(500)
+    lr, b1, b2, eps = 1e-2, 0.9, 0.999, 1e-8
+    for t in range(1, 51):
+        g = r.normal(0, 1, 500).astype(np.float32)
+        oracle.adam_step(p, g, m, v, lr, b1, b2, eps, t)
+        md = b1 * md + (1 - b1) * g
+        vd = b2 * vd + (1 - b2) * g.astype(np.float64) ** 2
+        pd -= lr * np.sqrt(1 - b2 ** t) / (1 - b1 ** t) * md / (np.sqrt(vd) + eps)
+    assert np.allclose(p, pd, atol=2e-5)

@@ -37,13 +37,20 @@ SIGNATURES = {
     "xad_host_chain_forward_backward_f32": [_sz] + [_vp] * 13 + [_int],
     "xad_host_chain_forward_backward_f64": [_sz] + [_vp] * 13 + [_int],
     "xad_accumulate_chain_gradients_f32": [_int, _sz] + [_vp] * 8 + [_int, _vp],
+    "xad_splat_create": [_int, _int, _int, _sz, ctypes.POINTER(_vp)],
+    "xad_splat_destroy": [_vp],
+    "xad_splat_forward": [_vp, _vp, _vp, _vp, _vp],
+    "xad_splat_step": [_vp, _vp, _vp, _vp, _vp, _vp, ctypes.POINTER(ctypes.c_double), _vp],
+    "xad_splat_set_profiling": [_vp, _int],
+    "xad_splat_get_stats": [_vp, ctypes.POINTER(_u64), ctypes.POINTER(ctypes.c_uint32), ctypes.POINTER(_flt)],
+    "xad_adam_step_f32": [_sz, _int, _vp, _vp, _vp, _vp, ctypes.POINTER(_flt), _flt, _flt, _flt, _int, _vp],
     "xad_rng_zipf_i32": [_vp, _sz, _u64, _u64, _int, ctypes.c_double, _vp],
     "xad_rng_uniform_f32": [_vp, _sz, _u64, _u64, _flt, _flt, _vp],
     "xad_rng_normal_f32": [_vp, _sz, _u64, _u64, _flt, _flt, _vp],
     "xad_host_rng_bits": [_vp, _sz, _u64, _u64, _u64],
     "xad_host_rng_uniform_f32": [_vp, _sz, _u64, _u64, _flt, _flt],
 }
-_RESTYPE = {"xad_last_error": ctypes.c_char_p}
+_RESTYPE = {"xad_last_error": ctypes.c_char_p, "xad_splat_destroy": None}
 
 
 def load():
