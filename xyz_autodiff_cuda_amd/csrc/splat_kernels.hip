@@ -12,6 +12,8 @@
 #include <operations/covariance_generation.cuh>
 #include <operations/mahalanobis_distance.cuh>
 
+#include <type_traits>
+
 #include "common.cuh"
 #include "splat.cuh"
 #include "splat_launch.cuh"
@@ -131,233 +133,313 @@ __device__ __forceinline__ int tile_of_block(int block, int tiles) {
     return t;  // may be >= tiles for the padding blocks of the last band
 }
 
-// alpha of one Gaussian at one pixel, before the clamp, through the library's
-// op logic (forward rules only): q = mahalanobis(pixel - centre; inv),
-// falloff = exp(-(q/2)), a = falloff * alpha0.
-struct PixelAlpha {
-    float q, falloff, a;
-};
-__device__ __forceinline__ PixelAlpha pixel_alpha(const Record& r, float px, float py) {
-    const float dx = px - r.cx, dy = py - r.cy;
-    PixelAlpha out;
-    out.q = op::detail_maha::quadratic_form<float>(dx, dy, r.a, r.b, r.c);
-    out.falloff = math::exp(-(out.q * 0.5f));
-    out.a = out.falloff * r.alpha0;
-    return out;
-}
+// ---------------------------------------------------------------------------
+// Compositing kernels.  One wavefront per tile; lane l owns the four
+// horizontally adjacent pixels x = 4 (l % 4) .. +3 of row y = l / 4.  Four
+// pixels per lane amortise everything that is per Gaussian (the LDS reads of
+// its record, and in the backward pass the wavefront reduction of its
+// gradient) over four times the arithmetic, and a one-wavefront block needs no
+// block barrier.
+//
+// The tile's list is staged through LDS 64 records at a time, in a form made
+// for the inner loop: the inverse covariance is pre-multiplied by
+// -log2(e)/2 so that the falloff exp(-q/2) is a single v_exp_f32 of
+//     q' = a' dx^2 + b2' dx dy + c' dy^2,
+// the graph  q = mahalanobis(pixel - centre; inv), falloff = exp(-(q * 0.5)),
+// a = falloff * alpha0  of the reference kernel
+// (examples/mini-gaussian-splatting/gaussian_splatting_kernel.cu:45-55) in fused form.
+constexpr int kLanePixels = 4;
+constexpr int kChunk = 64;
+constexpr float kHalfLog2e = 0.72134752044448170368f;  // log2(e) / 2
 
-__device__ __forceinline__ Record load_record(const Record* __restrict__ records, std::uint32_t g) {
+struct alignas(16) Staged {
+    float cx, cy, a_s, b2_s;          // centre; a' and 2b'
+    float c_s, alpha0, red, green;    // c'; sigmoid(opacity); colour
+    float blue, a, b, c;              // colour; inverse covariance as stored
+};
+static_assert(sizeof(Staged) == 48, "Staged must be three float4");
+
+__device__ __forceinline__ Staged stage_record(const Record* __restrict__ records, std::uint32_t g) {
     const float4* src = reinterpret_cast<const float4*>(records + g);
     const float4 v0 = src[0], v1 = src[1], v2 = src[2];
-    Record r;
-    r.cx = v0.x; r.cy = v0.y; r.a = v0.z; r.b = v0.w;
-    r.c = v1.x; r.red = v1.y; r.green = v1.z; r.blue = v1.w;
-    r.alpha0 = v2.x; r.pad0 = r.pad1 = r.pad2 = 0.f;
-    return r;
+    Staged s;
+    s.cx = v0.x;
+    s.cy = v0.y;
+    s.a = v0.z;
+    s.b = v0.w;
+    s.c = v1.x;
+    s.red = v1.y;
+    s.green = v1.z;
+    s.blue = v1.w;
+    s.alpha0 = v2.x;
+    s.a_s = -kHalfLog2e * s.a;
+    s.b2_s = -2.f * kHalfLog2e * s.b;
+    s.c_s = -kHalfLog2e * s.c;
+    return s;
 }
 
-// ---------------------------------------------------------------------------
-// Compositing forward: one 256-lane block per tile, one lane per pixel.  The
-// tile's list is staged through LDS 256 records at a time; every lane then
-// reads the same record at the same time (an LDS broadcast).
-__global__ void __launch_bounds__(kTilePixels) render_forward_kernel(
+__device__ __forceinline__ float falloff_of(const Staged& r, float dx, float dy) {
+    const float t = ::fmaf(r.b2_s, dy, r.a_s * dx);
+    const float q_scaled = ::fmaf(r.c_s * dy, dy, t * dx);
+    return math::fp32::exp2_raw(q_scaled);
+}
+
+__device__ __forceinline__ std::uint32_t wave_max(std::uint32_t v) {
+    // 64-lane maximum through the LDS crossbar-free DPP path: rows, then row heads
+    auto step = [](std::uint32_t x, auto ctrl) {
+        const std::uint32_t other = static_cast<std::uint32_t>(
+            __builtin_amdgcn_update_dpp(0, static_cast<int>(x), decltype(ctrl)::value, 0xF, 0xF, true));
+        return x > other ? x : other;
+    };
+    v = step(v, std::integral_constant<int, 0xB1>{});
+    v = step(v, std::integral_constant<int, 0x4E>{});
+    v = step(v, std::integral_constant<int, 0x141>{});
+    v = step(v, std::integral_constant<int, 0x140>{});
+    const std::uint32_t r0 = __builtin_amdgcn_readlane(static_cast<int>(v), 0);
+    const std::uint32_t r1 = __builtin_amdgcn_readlane(static_cast<int>(v), 16);
+    const std::uint32_t r2 = __builtin_amdgcn_readlane(static_cast<int>(v), 32);
+    const std::uint32_t r3 = __builtin_amdgcn_readlane(static_cast<int>(v), 48);
+    const std::uint32_t m01 = r0 > r1 ? r0 : r1, m23 = r2 > r3 ? r2 : r3;
+    return m01 > m23 ? m01 : m23;
+}
+
+__global__ void __launch_bounds__(kChunk) render_forward_kernel(
     int width, int height, int tiles_x, int tiles, const std::uint32_t* __restrict__ range_begin,
     const std::uint32_t* __restrict__ range_end, const std::uint32_t* __restrict__ sorted_ids,
     const Record* __restrict__ records, float* __restrict__ image, float* __restrict__ final_T,
     std::uint32_t* __restrict__ n_contrib) {
-    __shared__ Record staged[kTilePixels];
+    __shared__ Staged staged[kChunk];
     const int tile = tile_of_block(blockIdx.x, tiles);
     if (tile >= tiles) return;
-    const int tx = tile % tiles_x, ty = tile / tiles_x;
-    const int lx = threadIdx.x % kTile, ly = threadIdx.x / kTile;
-    const int x = tx * kTile + lx, y = ty * kTile + ly;
-    const bool inside = x < width && y < height;
-    const float px = static_cast<float>(x), py = static_cast<float>(y);
+    const int lane = threadIdx.x;
+    const int x0 = (tile % tiles_x) * kTile + (lane & 3) * kLanePixels;
+    const int y = (tile / tiles_x) * kTile + (lane >> 2);
+    const float py = static_cast<float>(y);
 
     const std::uint32_t first = range_begin[tile], last = range_end[tile];
-    float T = 1.f, red = 0.f, green = 0.f, blue = 0.f;
-    std::uint32_t used = 0;
-    bool done = !inside;
+    float T[kLanePixels], red[kLanePixels], green[kLanePixels], blue[kLanePixels];
+    std::uint32_t used[kLanePixels];
+    bool done[kLanePixels];
+#pragma unroll
+    for (int p = 0; p < kLanePixels; ++p) {
+        T[p] = 1.f;
+        red[p] = green[p] = blue[p] = 0.f;
+        used[p] = 0;
+        done[p] = !(x0 + p < width && y < height);
+    }
 
-    for (std::uint32_t base = first; base < last; base += kTilePixels) {
+    for (std::uint32_t base = first; base < last; base += kChunk) {
         __syncthreads();
-        const std::uint32_t mine = base + threadIdx.x;
-        if (mine < last) staged[threadIdx.x] = load_record(records, sorted_ids[mine]);
+        if (base + lane < last) staged[lane] = stage_record(records, sorted_ids[base + lane]);
         __syncthreads();
-        const int count = static_cast<int>(last - base < kTilePixels ? last - base : kTilePixels);
-        if (!done) {
-            for (int j = 0; j < count; ++j) {
-                if (T < kMinTransmittance) {
-                    done = true;
-                    break;
-                }
-                const Record& r = staged[j];
-                const PixelAlpha pa = pixel_alpha(r, px, py);
-                const float alpha = pa.a > kAlphaMax ? kAlphaMax : pa.a;
-                const float weight = T * alpha;
-                red += weight * r.red;
-                green += weight * r.green;
-                blue += weight * r.blue;
-                T *= 1.f - alpha;
-                used = base - first + j + 1;
+        const int count = static_cast<int>(last - base < kChunk ? last - base : kChunk);
+        for (int j = 0; j < count; ++j) {
+            const Staged r = staged[j];
+            const float dy = py - r.cy;
+#pragma unroll
+            for (int p = 0; p < kLanePixels; ++p) {
+                // a pixel stops, for good, before the first Gaussian it meets with T below the threshold
+                done[p] = done[p] || T[p] < kMinTransmittance;
+                const float dx = static_cast<float>(x0 + p) - r.cx;
+                const float a = falloff_of(r, dx, dy) * r.alpha0;
+                const float alpha = done[p] ? 0.f : (a > kAlphaMax ? kAlphaMax : a);
+                const float weight = T[p] * alpha;
+                red[p] = ::fmaf(weight, r.red, red[p]);
+                green[p] = ::fmaf(weight, r.green, green[p]);
+                blue[p] = ::fmaf(weight, r.blue, blue[p]);
+                T[p] *= 1.f - alpha;
+                used[p] = done[p] ? used[p] : base - first + j + 1;
             }
         }
-        if (__syncthreads_and(done)) break;
+        const bool all_done = done[0] && done[1] && done[2] && done[3];
+        if (accumulate::wave::ballot(!all_done) == 0) break;
     }
-    if (inside) {
-        const std::size_t p = static_cast<std::size_t>(y) * width + x;
-        image[p * 3 + 0] = red;
-        image[p * 3 + 1] = green;
-        image[p * 3 + 2] = blue;
-        final_T[p] = T;
-        n_contrib[p] = used;
+#pragma unroll
+    for (int p = 0; p < kLanePixels; ++p) {
+        if (x0 + p < width && y < height) {
+            const std::size_t at = static_cast<std::size_t>(y) * width + x0 + p;
+            image[at * 3 + 0] = red[p];
+            image[at * 3 + 1] = green[p];
+            image[at * 3 + 2] = blue[p];
+            final_T[at] = T[p];
+            n_contrib[at] = used[p];
+        }
     }
 }
 
-// ---------------------------------------------------------------------------
-// Compositing backward: same tiling, lists walked back to front.  For every
-// (pixel, Gaussian) the lane computes d loss / d (centre, inverse covariance,
-// colour, alpha0); the nine values are summed over the 64 lanes of each
-// wavefront with DPP, the four wavefront sums are combined through LDS, and one
-// lane per Gaussian adds the block's totals to the global accumulator: one
-// global atomic per (tile, Gaussian, field).
-__global__ void __launch_bounds__(kTilePixels) render_backward_kernel(
+// Sum of nine per-lane values over the wavefront, cheaper than nine separate
+// reductions.  v[0..7] go through a reduce-scatter: at each of the first three
+// steps a lane hands half of its values to its partner (lane ^ 1, ^ 2, ^ 4) and
+// adds the partner's copies of the half it keeps, so after 4 + 2 + 1 exchanges
+// lane l holds value l % 8 summed over its group of eight lanes; one rotation
+// by eight completes the row of 16.  v[8] takes the ordinary four row steps.
+// Result: in every row of 16 lanes, lane m < 8 holds the row's sum of v[m] and
+// lane 8 that of v[8]; the four rows are added by whoever reads them.
+__device__ __forceinline__ float reduce_scatter9(const float (&v)[9], int lane) {
+    const bool b0 = lane & 1, b1 = lane & 2, b2 = lane & 4;
+    float w[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const float keep = b0 ? v[2 * i + 1] : v[2 * i];
+        const float send = b0 ? v[2 * i] : v[2 * i + 1];
+        w[i] = keep + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, send), 0xB1, 0xF, 0xF, true));
+    }
+    float u[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const float keep = b1 ? w[2 * i + 1] : w[2 * i];
+        const float send = b1 ? w[2 * i] : w[2 * i + 1];
+        u[i] = keep + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, send), 0x4E, 0xF, 0xF, true));
+    }
+    const float keep = b2 ? u[1] : u[0];
+    const float send = b2 ? u[0] : u[1];
+    // lane ^ 4: a shift by four towards lower lanes feeds banks 0 and 2, towards higher lanes banks 1 and 3
+    int other = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, send), 0x104, 0xF, 0x5, false);   // row_shl:4
+    other = __builtin_amdgcn_update_dpp(other, __builtin_bit_cast(int, send), 0x114, 0xF, 0xA, false);    // row_shr:4
+    float t = keep + __builtin_bit_cast(float, other);
+    t = accumulate::wave::dpp_add<0x128>(t);  // row_ror:8
+
+    float x = v[8];
+    x = accumulate::wave::dpp_add<0xB1>(x);
+    x = accumulate::wave::dpp_add<0x4E>(x);
+    x = accumulate::wave::dpp_add<0x141>(x);
+    x = accumulate::wave::dpp_add<0x140>(x);
+    return (lane & 8) ? x : t;
+}
+
+// Compositing backward.  Lists are walked back to front.  For every Gaussian
+// each lane adds up, over its four pixels, the nine sums that determine
+// d loss / d record:
+//   S_x, S_y, S_xx, S_xy, S_yy = sum of g_q {dx, dy, dx^2, dx dy, dy^2},  g_q = d loss / d q
+//   the three colour gradients, and d loss / d alpha0
+// (the Mahalanobis backward rule, d centre = -g_q (2a dx + 2b dy, 2b dx + 2c dy),
+// d inv = g_q (dx^2, 2 dx dy, dy^2), is linear in those sums, so it is applied
+// once per Gaussian instead of once per pixel).  The nine values are reduced
+// over the wavefront by reduce_scatter9 and parked in LDS; after each chunk of
+// 64 Gaussians lane j finishes Gaussian j and adds its nine record gradients to
+// the global accumulator: one global atomic per (tile, Gaussian, field).
+__global__ void __launch_bounds__(kChunk) render_backward_kernel(
     int width, int height, int tiles_x, int tiles, const std::uint32_t* __restrict__ range_begin,
     const std::uint32_t* __restrict__ range_end, const std::uint32_t* __restrict__ sorted_ids,
     const Record* __restrict__ records, const float* __restrict__ image, const float* __restrict__ target,
     const float* __restrict__ final_T, const std::uint32_t* __restrict__ n_contrib, float* __restrict__ record_grads,
     double* __restrict__ loss) {
-    constexpr int kWaves = kTilePixels / 64;
-    __shared__ Record staged[kTilePixels];
-    __shared__ std::uint32_t staged_id[kTilePixels];
-    __shared__ float partial[kWaves][kTilePixels][kRecordGrads];  // [wave][list entry][field]
-    __shared__ std::uint32_t block_max_used;
-    __shared__ double wave_loss[kWaves];
+    __shared__ Staged staged[kChunk];
+    __shared__ std::uint32_t staged_id[kChunk];
+    __shared__ float parked[kChunk][4][9];  // [list entry][row of 16 lanes][value]
 
     const int tile = tile_of_block(blockIdx.x, tiles);
     if (tile >= tiles) return;
-    const int tx = tile % tiles_x, ty = tile / tiles_x;
-    const int lx = threadIdx.x % kTile, ly = threadIdx.x / kTile;
-    const int x = tx * kTile + lx, y = ty * kTile + ly;
-    const bool inside = x < width && y < height;
-    const float px = static_cast<float>(x), py = static_cast<float>(y);
-    const int wave = threadIdx.x / 64;
-    const std::size_t p = static_cast<std::size_t>(y) * width + x;
+    const int lane = threadIdx.x;
+    const int x0 = (tile % tiles_x) * kTile + (lane & 3) * kLanePixels;
+    const int y = (tile / tiles_x) * kTile + (lane >> 2);
+    const float py = static_cast<float>(y);
 
-    float dC[3] = {0.f, 0.f, 0.f};
-    float T = 1.f;
-    std::uint32_t used = 0;
+    float dC[kLanePixels][3], T[kLanePixels], behind[kLanePixels][3], last_alpha[kLanePixels];
+    std::uint32_t used[kLanePixels];
     float my_loss = 0.f;
-    if (inside) {
+    std::uint32_t my_max = 0;
 #pragma unroll
-        for (int c = 0; c < 3; ++c) {
-            const float d = image[p * 3 + c] - target[p * 3 + c];
-            my_loss += d * d;
-            dC[c] = 2.f * d;
+    for (int p = 0; p < kLanePixels; ++p) {
+        T[p] = 1.f;
+        used[p] = 0;
+        last_alpha[p] = 0.f;
+#pragma unroll
+        for (int c = 0; c < 3; ++c) dC[p][c] = behind[p][c] = 0.f;
+        if (x0 + p < width && y < height) {
+            const std::size_t at = static_cast<std::size_t>(y) * width + x0 + p;
+#pragma unroll
+            for (int c = 0; c < 3; ++c) {
+                const float d = image[at * 3 + c] - target[at * 3 + c];
+                my_loss = ::fmaf(d, d, my_loss);
+                dC[p][c] = 2.f * d;
+            }
+            T[p] = final_T[at];
+            used[p] = n_contrib[at];
+            my_max = used[p] > my_max ? used[p] : my_max;
         }
-        T = final_T[p];
-        used = n_contrib[p];
     }
-    // loss: per-wavefront DPP sum, then one fp64 atomic per block
     {
-        const float s = accumulate::wave::sum(my_loss);
-        if (threadIdx.x % 64 == 0) wave_loss[wave] = static_cast<double>(s);
-        if (threadIdx.x == 0) block_max_used = 0;
-        __syncthreads();
-        atomicMax(&block_max_used, used);
-        if (threadIdx.x == 0) {
-            double total = 0.0;
-            for (int w = 0; w < kWaves; ++w) total += wave_loss[w];
-            if (total != 0.0) detail::atomic_add(loss, total);
-        }
-        __syncthreads();
+        const float tile_loss = accumulate::wave::sum(my_loss);
+        if (lane == 0 && tile_loss != 0.f) detail::atomic_add(loss, static_cast<double>(tile_loss));
     }
-    const std::uint32_t first = range_begin[tile];
-    const std::uint32_t deepest = block_max_used;  // entries [0, deepest) of the list were used by some pixel
+    const std::uint32_t deepest = wave_max(my_max);  // entries [0, deepest) were composited by some pixel
     if (deepest == 0) return;
+    const std::uint32_t first = range_begin[tile];
+    float last_col[3] = {0.f, 0.f, 0.f};
 
-    float behind[3] = {0.f, 0.f, 0.f}, last_col[3] = {0.f, 0.f, 0.f};
-    float last_alpha = 0.f;
-
-    const std::uint32_t chunks = (deepest + kTilePixels - 1) / kTilePixels;
-    for (std::uint32_t chunk = chunks; chunk-- > 0;) {
-        const std::uint32_t chunk_first = chunk * kTilePixels;  // list position of staged[0]
-        const int count = static_cast<int>(deepest - chunk_first < kTilePixels ? deepest - chunk_first : kTilePixels);
+    for (std::uint32_t chunk = (deepest + kChunk - 1) / kChunk; chunk-- > 0;) {
+        const std::uint32_t chunk_first = chunk * kChunk;
+        const int count = static_cast<int>(deepest - chunk_first < kChunk ? deepest - chunk_first : kChunk);
         __syncthreads();
-        if (static_cast<int>(threadIdx.x) < count) {
-            const std::uint32_t id = sorted_ids[first + chunk_first + threadIdx.x];
-            staged_id[threadIdx.x] = id;
-            staged[threadIdx.x] = load_record(records, id);
+        if (lane < count) {
+            const std::uint32_t id = sorted_ids[first + chunk_first + lane];
+            staged_id[lane] = id;
+            staged[lane] = stage_record(records, id);
         }
         __syncthreads();
 
         for (int j = count - 1; j >= 0; --j) {
             const std::uint32_t position = chunk_first + j;
-            const bool active = position < used;  // `used` is 0 for lanes outside the image
-            if (accumulate::wave::ballot(active) == 0) {
-                // no pixel of this wavefront composited this Gaussian
-                if (threadIdx.x % 64 < kRecordGrads) partial[wave][j][threadIdx.x % 64] = 0.f;
-                continue;
-            }
-            float g[kRecordGrads] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-            if (active) {
-                const Record& r = staged[j];
-                const PixelAlpha pa = pixel_alpha(r, px, py);
-                const float alpha = pa.a > kAlphaMax ? kAlphaMax : pa.a;
-                T = T / (1.f - alpha);
-                const float col[3] = {r.red, r.green, r.blue};
+            const Staged r = staged[j];
+            const float dy = py - r.cy;
+            const float g_q_scale = -0.5f * r.alpha0;
+            float v[9] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int p = 0; p < kLanePixels; ++p) {
+                // A pixel is idle until the walk reaches the last Gaussian it composited, and
+                // active from there on.  While idle, alpha = 0 leaves T, `behind` and
+                // last_alpha at their initial values, so no branch is needed.
+                const bool active = position < used[p];
+                const float dx = static_cast<float>(x0 + p) - r.cx;
+                const float falloff = falloff_of(r, dx, dy);
+                const float a = falloff * r.alpha0;
+                const bool clamped = a > kAlphaMax;
+                const float alpha = active ? (clamped ? kAlphaMax : a) : 0.f;
+                T[p] = T[p] * __builtin_amdgcn_rcpf(1.f - alpha);  // transmittance in front of this Gaussian
                 float d_alpha = 0.f;
+                const float col[3] = {r.red, r.green, r.blue};
+                const float weight = alpha * T[p];
 #pragma unroll
                 for (int c = 0; c < 3; ++c) {
-                    behind[c] = last_alpha * last_col[c] + (1.f - last_alpha) * behind[c];
-                    d_alpha += (col[c] - behind[c]) * dC[c];
-                    g[5 + c] = alpha * T * dC[c];
-                    last_col[c] = col[c];
+                    behind[p][c] = ::fmaf(last_alpha[p], last_col[c] - behind[p][c], behind[p][c]);
+                    d_alpha = ::fmaf(col[c] - behind[p][c], dC[p][c], d_alpha);
+                    v[5 + c] = ::fmaf(weight, dC[p][c], v[5 + c]);
                 }
-                d_alpha *= T;
-                last_alpha = alpha;
-                if (!(pa.a > kAlphaMax)) {
-                    // a = falloff * alpha0; falloff = exp(-(q/2)); q = mahalanobis(pixel, centre, inv):
-                    // the library's backward rules, applied to thread-local operands
-                    g[8] = d_alpha * pa.falloff;
-                    const float g_q = -0.5f * (d_alpha * r.alpha0 * pa.falloff);
-                    Variable<2, float> centre;
-                    centre[0] = r.cx;
-                    centre[1] = r.cy;
-                    Variable<3, float> inv;
-                    inv[0] = r.a;
-                    inv[1] = r.b;
-                    inv[2] = r.c;
-                    Variable<1, float> q_out;
-                    q_out.add_grad(0, g_q);
-                    const op::MahalanobisDistanceWithCenterLogic<Variable<2, float>, Variable<3, float>> rule(px, py);
-                    rule.backward(q_out, centre, inv);
-                    g[0] = centre.grad(0);
-                    g[1] = centre.grad(1);
-                    g[2] = inv.grad(0);
-                    g[3] = inv.grad(1);
-                    g[4] = inv.grad(2);
-                }
+                last_alpha[p] = alpha;
+                const float through = (active && !clamped) ? d_alpha * T[p] * falloff : 0.f;  // d loss / d alpha0
+                v[8] += through;
+                const float g_q = through * g_q_scale;
+                const float gx = g_q * dx, gy = g_q * dy;
+                v[0] += gx;
+                v[1] += gy;
+                v[2] = ::fmaf(gx, dx, v[2]);
+                v[3] = ::fmaf(gx, dy, v[3]);
+                v[4] = ::fmaf(gy, dy, v[4]);
             }
-            // level 1: wavefront sums
-#pragma unroll
-            for (int k = 0; k < kRecordGrads; ++k) {
-                const float s = accumulate::wave::sum(g[k]);
-                if (threadIdx.x % 64 == 0) partial[wave][j][k] = s;
-            }
+            last_col[0] = r.red;
+            last_col[1] = r.green;
+            last_col[2] = r.blue;
+            const float mine = reduce_scatter9(v, lane);
+            if ((lane & 15) < 9) parked[j][lane >> 4][lane & 15] = mine;
         }
         __syncthreads();
-        // level 2 + 3: lane j combines the four wavefront sums of list entry j and
-        // adds them to the Gaussian's accumulator row
-        if (static_cast<int>(threadIdx.x) < count) {
-            float* row = record_grads + static_cast<std::size_t>(staged_id[threadIdx.x]) * kRecordGrads;
+        if (lane < count) {
+            float s[9];
 #pragma unroll
-            for (int k = 0; k < kRecordGrads; ++k) {
-                float s = 0.f;
+            for (int k = 0; k < 9; ++k) s[k] = (parked[lane][0][k] + parked[lane][1][k]) + (parked[lane][2][k] + parked[lane][3][k]);
+            const Staged r = staged[lane];
+            float* row = record_grads + static_cast<std::size_t>(staged_id[lane]) * kRecordGrads;
+            const float out[kRecordGrads] = {
+                -(2.f * r.a * s[0] + 2.f * r.b * s[1]),  // d centre x
+                -(2.f * r.b * s[0] + 2.f * r.c * s[1]),  // d centre y
+                s[2], 2.f * s[3], s[4],                  // d inverse covariance
+                s[5], s[6], s[7],                        // d colour
+                s[8],                                    // d alpha0
+            };
 #pragma unroll
-                for (int w = 0; w < kWaves; ++w) s += partial[w][threadIdx.x][k];
-                if (s != 0.f) detail::atomic_add(row + k, s);
-            }
+            for (int k = 0; k < kRecordGrads; ++k)
+                if (out[k] != 0.f) detail::atomic_add(row + k, out[k]);
         }
     }
 }
@@ -439,7 +521,7 @@ int launch_render_forward(hipStream_t s, int width, int height, const std::uint3
                           const std::uint32_t* range_end, const std::uint32_t* sorted_ids, const Record* records,
                           float* image, float* final_T, std::uint32_t* n_contrib) {
     const int tiles_x = (width + kTile - 1) / kTile, tiles = tiles_x * ((height + kTile - 1) / kTile);
-    hipLaunchKernelGGL(render_forward_kernel, dim3(padded_tile_blocks(tiles)), dim3(kTilePixels), 0, s, width, height,
+    hipLaunchKernelGGL(render_forward_kernel, dim3(padded_tile_blocks(tiles)), dim3(kChunk), 0, s, width, height,
                        tiles_x, tiles, range_begin, range_end, sorted_ids, records, image, final_T, n_contrib);
     XAD_HIP_TRY(hipGetLastError());
     return XAD_OK;
@@ -450,7 +532,7 @@ int launch_render_backward(hipStream_t s, int width, int height, const std::uint
                            const float* image, const float* target, const float* final_T,
                            const std::uint32_t* n_contrib, float* record_grads, double* loss) {
     const int tiles_x = (width + kTile - 1) / kTile, tiles = tiles_x * ((height + kTile - 1) / kTile);
-    hipLaunchKernelGGL(render_backward_kernel, dim3(padded_tile_blocks(tiles)), dim3(kTilePixels), 0, s, width, height,
+    hipLaunchKernelGGL(render_backward_kernel, dim3(padded_tile_blocks(tiles)), dim3(kChunk), 0, s, width, height,
                        tiles_x, tiles, range_begin, range_end, sorted_ids, records, image, target, final_T, n_contrib,
                        record_grads, loss);
     XAD_HIP_TRY(hipGetLastError());
