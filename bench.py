@@ -20,6 +20,9 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published
+# HBM bytes per evaluation of the chain kernel, from FETCH_SIZE / WRITE_SIZE counter
+# passes scaled by a copy of known size (profiles/chain_single_kernel_hbm_traffic.md)
+MEASURED_TRAFFIC_BYTES_PER_EVAL = 52.003
 N_FULL = 64 * 1024 * 1024
 
 
@@ -114,6 +117,83 @@ def accumulate_report(ins, seed, with_oracle):
     return out
 
 
+def splat_report(with_oracle, iters=30):
+    """Configs 4 and 5: one training iteration = forward + backward + Adam (lr 1e-2).
+    Reports iterations/s, the per-kernel time split, pair statistics, and the CPU
+    oracle's time for the same iteration on the host cores."""
+    import numpy as np
+    import torch
+
+    from xyz_autodiff_cuda_amd import splat
+
+    dev = torch.device("cuda:0")
+    out = {}
+    for name, G, W, H, scale in (("config4_10k_512", 10_000, 512, 512, (1.0, 20.0)),
+                                 ("config5_200k_2048", 200_000, 2048, 2048, (0.5, 40.0))):
+        target = splat.synthetic_target(G, W, H, seed=77, scale_px=scale, noise=0.02)
+        params, depth = splat.synthetic_scene(G, W, H, seed=1234, scale_px=scale)
+        start_params = params.clone()
+        ctx = splat.SplatContext(W, H, G, pair_capacity_hint=9_000_000 if G > 50_000 else 0)
+        m, v = torch.zeros_like(params), torch.zeros_like(params)
+        image = torch.empty(H, W, 3, device=dev)
+        grads = torch.empty(9, G, device=dev)
+        _, _, first_loss = ctx.step(params, depth, target, image, grads)
+        for it in range(1, 4):
+            ctx.step(params, depth, target, image, grads, want_loss=False)
+            splat.adam_step(params, grads, m, v, 1e-2, it)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for it in range(4, 4 + iters):
+            ctx.step(params, depth, target, image, grads, want_loss=False)
+            splat.adam_step(params, grads, m, v, 1e-2, it)
+        torch.cuda.synchronize()
+        per_iter = (time.perf_counter() - t0) / iters
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for it in range(10):
+            splat.adam_step(params, grads, m, v, 1e-2, 100 + it)
+        b.record()
+        torch.cuda.synchronize()
+        adam_ms = a.elapsed_time(b) / 10
+        ctx.set_profiling(True)
+        acc = None
+        for _ in range(5):
+            ctx.step(params, depth, target, image, grads, want_loss=False)
+            ms = ctx.stats()["stage_ms"]
+            acc = ms if acc is None else {k: acc[k] + ms[k] for k in ms}
+        ctx.set_profiling(False)
+        _, _, last_loss = ctx.step(params, depth, target, image, grads)
+        stats = ctx.stats(longest_list=True)
+        tiles = ((W + 15) // 16) * ((H + 15) // 16)
+        entry = {
+            "gaussians": G, "image": [W, H], "iters_per_s": 1.0 / per_iter, "ms_per_iter": per_iter * 1e3,
+            "stage_ms": {**{k: v / 5 for k, v in acc.items()}, "adam": adam_ms},
+            "pairs": stats["pairs"], "mean_list": stats["pairs"] / tiles, "longest_list": stats["longest_list"],
+            "global_atomics_per_iter": {"after_block_pre_reduction": stats["pairs"] * 9 + tiles,
+                                        "per_pixel_pair_naive": int(stats["pairs"]) * 256 * 9},
+            "loss_first": first_loss, "loss_after_%d_iters" % (iters + 8): last_loss,
+        }
+        if with_oracle:
+            from tests import _oracle
+
+            oracle = _oracle.load()
+            hp, hd, ht = start_params.cpu().numpy(), depth.cpu().numpy(), target.cpu().numpy()
+            t0 = time.perf_counter()
+            ref = oracle.splat_step(W, H, hp, hd, ht, np.float32)
+            cpu_s = time.perf_counter() - t0
+            hm, hv = np.zeros_like(hp), np.zeros_like(hp)
+            t0 = time.perf_counter()
+            oracle.adam_step(hp, ref["grads"], hm, hv, 1e-2, 0.9, 0.999, 1e-8, 1)
+            cpu_s += time.perf_counter() - t0
+            entry["cpu_oracle"] = {"s_per_iter": cpu_s, "iters_per_s": 1.0 / cpu_s, "cores": oracle.max_threads(),
+                                   "stage_s": ref["seconds"], "sample": "one full iteration"}
+            entry["speedup_vs_cpu"] = cpu_s / per_iter
+            entry["first_loss_matches_cpu"] = abs(first_loss - ref["loss"]) <= 1e-5 * ref["loss"]
+        ctx.close()
+        out[name] = entry
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -122,6 +202,8 @@ def main():
     ap.add_argument("--n", type=int, default=N_FULL, help="problems per step (default: the full 64 Mi)")
     ap.add_argument("--seed", type=int, default=1234)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs (profiling runs)")
+    ap.add_argument("--counter-probe", action="store_true",
+                    help="launch only a 256 Mi-float copy and three chain passes, then exit (for rocprofv3 --pmc runs)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (got --gpus %d)" % args.gpus)
@@ -138,6 +220,15 @@ def main():
     outs = [torch.empty(n, dtype=torch.float32, device=dev) for _ in range(7)]
     rng.chain_inputs_(ins, args.seed)
     torch.cuda.synchronize()
+
+    if args.counter_probe:
+        # known traffic first (1 GiB read + 1 GiB written), then the kernel under study
+        chain.stream_copy(torch.cat(ins[:4]), torch.cat(outs[:4]))
+        for _ in range(3):
+            chain.forward_backward(ins, outs)
+        torch.cuda.synchronize()
+        print(json.dumps({"counter_probe": True, "n": n, "copy_floats": 4 * n}))
+        return
 
     for _ in range(args.warmup):
         chain.forward_backward(ins, outs)
@@ -197,7 +288,7 @@ def main():
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBPS,
-            "traffic": None,
+            "traffic": MEASURED_TRAFFIC_BYTES_PER_EVAL * n,
             "kernel": "chain_single_kernel",
             "kernel_ms_avg": avg_kernel_s * 1e3,
             "kernel_ms_min": min(kernel_ms),
@@ -211,6 +302,9 @@ def main():
         host_inputs = [t[:sample_n].cpu().numpy() for t in ins]
         record["cpu_baseline"] = cpu_baseline(host_inputs)
         record["host_templates"] = host_templates(host_inputs)
+    del ins, outs
+    torch.cuda.empty_cache()
+    record["splat"] = splat_report(with_oracle=not args.no_cpu)
     print(json.dumps(record))
 
 

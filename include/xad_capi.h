@@ -73,6 +73,11 @@ int xad_chain_forward_backward_f32_layout(size_t n,
                                           float* d_o, float* d_px, float* d_py,
                                           int problems_per_lane, void* stream);
 
+/* dst[i] = src[i] for n floats on the device, with the access pattern of the
+ * kernel above: a copy of known size to calibrate counters and bandwidth against.
+ * No counterpart in the reference. */
+int xad_stream_copy_f32(size_t n, const float* src, float* dst, void* stream);
+
 /* The same graph from the same templates, compiled for the host and run on
  * `num_threads` host threads (<= 0: all hardware threads).  Host pointers.
  * Synchronous.  This is the "host-core run of the per-thread templates"; GPU

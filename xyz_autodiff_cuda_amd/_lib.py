@@ -34,6 +34,7 @@ SIGNATURES = {
     "xad_abi_version": [],
     "xad_chain_forward_backward_f32": [_sz] + [_vp] * 13 + [_vp],
     "xad_chain_forward_backward_f32_layout": [_sz] + [_vp] * 13 + [_int, _vp],
+    "xad_stream_copy_f32": [_sz, _vp, _vp, _vp],
     "xad_host_chain_forward_backward_f32": [_sz] + [_vp] * 13 + [_int],
     "xad_host_chain_forward_backward_f64": [_sz] + [_vp] * 13 + [_int],
     "xad_accumulate_chain_gradients_f32": [_int, _sz] + [_vp] * 8 + [_int, _vp],

@@ -76,3 +76,17 @@ def host_forward_backward(inputs, dtype=np.float32, num_threads=0):
     status = fn(n, *[a.ctypes.data for a in arrays], *[a.ctypes.data for a in outs], int(num_threads))
     _lib.check(status, fn.__name__)
     return outs
+
+
+def stream_copy(src, dst, stream=None):
+    """dst[:] = src on the GPU with the chain kernel's access pattern (calibration yardstick)."""
+    import torch
+
+    n = src.numel()
+    _require_cuda_f32(src, "src", n)
+    _require_cuda_f32(dst, "dst", n)
+    s = stream if stream is not None else torch.cuda.current_stream(src.device)
+    with torch.cuda.device(src.device):
+        st = _lib.load().xad_stream_copy_f32(n, src.data_ptr(), dst.data_ptr(), s.cuda_stream)
+    _lib.check(st, "xad_stream_copy_f32")
+    return dst

@@ -74,6 +74,14 @@ __global__ void __launch_bounds__(kSingleBlock) chain_single_kernel(ChainBuffers
     for (int a = 0; a < 7; ++a) __builtin_nontemporal_store(y[a], buf.out[a] + i);
 }
 
+// Plain copy with the chain kernel's access pattern (4 bytes per lane, non-temporal):
+// the yardstick that hardware counters and achievable bandwidth are scaled by.
+__global__ void __launch_bounds__(kSingleBlock) stream_copy_kernel(const float* __restrict__ src, float* __restrict__ dst,
+                                                                   std::size_t n) {
+    const std::size_t i = static_cast<std::size_t>(blockIdx.x) * kSingleBlock + threadIdx.x;
+    if (i < n) __builtin_nontemporal_store(__builtin_nontemporal_load(src + i), dst + i);
+}
+
 template <typename T>
 void host_chain_range(std::size_t begin, std::size_t end, const T* const* in, T* const* out) {
     for (std::size_t i = begin; i < end; ++i) {
@@ -162,6 +170,16 @@ extern "C" int xad_chain_forward_backward_f32_layout(std::size_t n, const float*
                                                      int problems_per_lane, void* stream) {
     const ChainBuffers buf{{sx, sy, theta, o, px, py}, {w, d_sx, d_sy, d_theta, d_o, d_px, d_py}};
     return launch_chain(n, buf, problems_per_lane, stream, "xad_chain_forward_backward_f32_layout");
+}
+
+extern "C" int xad_stream_copy_f32(std::size_t n, const float* src, float* dst, void* stream) {
+    if (n == 0) return XAD_OK;
+    XAD_REQUIRE(src && dst, "xad_stream_copy_f32: null array");
+    XAD_REQUIRE(n <= 0x7fffffffull * 64, "xad_stream_copy_f32: n = %zu exceeds the grid limit", n);
+    hipLaunchKernelGGL(stream_copy_kernel, dim3(xad::blocks_for(n, kSingleBlock)), dim3(kSingleBlock), 0,
+                       xad::as_stream(stream), src, dst, n);
+    XAD_HIP_TRY(hipGetLastError());
+    return XAD_OK;
 }
 
 extern "C" int xad_host_chain_forward_backward_f32(std::size_t n, const float* sx, const float* sy,
