@@ -10,9 +10,15 @@
 // temporaries (`a * b + c`) deliberately does not compile.
 // Same overload set as xyz-autodiff-cuda include/xyz_autodiff/variable_operators.cuh:23-79.
 // Include after the op headers whose factories it forwards to.
+//
+// One deliberate difference: `A * B` between two matrix views (DenseMatrix and
+// friends) is the matrix product of dense_matrix.cuh, never the element-wise
+// node.  With the reference's overload set the element-wise form silently wins
+// for two non-const square matrices of equal size once both headers are included.
 
 #include <concepts>
 
+#include <xyz_autodiff/concept/matrix.cuh>
 #include <xyz_autodiff/concept/variable.cuh>
 #include <xyz_autodiff/operations/binary/add_logic.cuh>
 #include <xyz_autodiff/operations/binary/div_logic.cuh>
@@ -53,9 +59,14 @@ XAD_SCALAR_OPERATOR(/, div_constant)
     }
 XAD_ELEMENTWISE_OPERATOR(+, add)
 XAD_ELEMENTWISE_OPERATOR(-, sub)
-XAD_ELEMENTWISE_OPERATOR(*, mul)
 XAD_ELEMENTWISE_OPERATOR(/, div)
 #undef XAD_ELEMENTWISE_OPERATOR
+
+template <typename Var1, typename Var2>
+    requires detail::SameShape<Var1, Var2> && (!(MatrixViewConcept<Var1> && MatrixViewConcept<Var2>))
+XAD_INLINE auto operator*(Var1& lhs, Var2& rhs) {
+    return op::mul(lhs, rhs);
+}
 
 template <DifferentiableVariableConcept Var, typename ConstArray>
     requires op::ArrayLikeConcept<ConstArray>

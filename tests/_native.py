@@ -1,0 +1,73 @@
+"""ctypes access to tests/native/libxad_api_tier.so (the API test tier)."""
+import ctypes
+import os
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "native", "libxad_api_tier.so")
+
+_lib = None
+
+# logic ids of xad_test_eval_logic: name -> (id, operand sizes, constants, outputs)
+LOGICS = {
+    "exp": (0, (3,), 0, 3), "sin": (1, (3,), 0, 3), "cos": (2, (3,), 0, 3), "sigmoid": (3, (3,), 0, 3),
+    "neg": (4, (3,), 0, 3), "squared": (5, (3,), 0, 3), "sum": (6, (4,), 0, 1), "l1_norm": (7, (4,), 0, 1),
+    "l2_norm": (8, (4,), 0, 1), "add_constant": (9, (3,), 1, 3), "sub_constant": (10, (3,), 1, 3),
+    "mul_constant": (11, (3,), 1, 3), "div_constant": (12, (3,), 1, 3), "const_add": (13, (3,), 3, 3),
+    "const_sub": (14, (3,), 3, 3), "sym_matrix2_inv": (15, (3,), 0, 3), "quaternion_to_rotation_matrix": (16, (4,), 0, 9),
+    "broadcast_logic": (17, (1,), 0, 4), "add": (18, (3, 3), 0, 3), "sub": (19, (3, 3), 0, 3), "mul": (20, (3, 3), 0, 3),
+    "div": (21, (3, 3), 0, 3), "matmul_2x2": (22, (4, 4), 0, 4), "matmul_3x3": (23, (9, 9), 0, 9),
+    "matvec_2x3": (24, (6, 3), 0, 2), "vecmat_3x2": (25, (3, 6), 0, 2), "generate_covariance_matrix": (26, (2, 1), 0, 4),
+    "matrix_to_covariance_3param": (27, (4,), 0, 3), "scale_rotation_to_covariance_3param": (28, (2, 1), 0, 3),
+    "mahalanobis_distance": (29, (2, 3), 0, 1), "mahalanobis_distance_with_center": (30, (2, 3), 2, 1),
+}
+
+
+def load():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise ImportError("tests/native/libxad_api_tier.so is not built; run `python tests/native/build.py`")
+        _lib = ctypes.CDLL(LIB_PATH)
+    return _lib
+
+
+def run_case(case_id, device=False):
+    lib = load()
+    out = np.zeros(lib.xad_test_case_capacity(), np.float64)
+    fn = lib.xad_test_run_case_device if device else lib.xad_test_run_case_host
+    n = fn(ctypes.c_int(case_id), out.ctypes.data_as(ctypes.c_void_p))
+    assert n >= 0, "case %d failed with %d" % (case_id, n)
+    return out[:n]
+
+
+def eval_logic(name, operands, constants=(), upstream=None, dtype=np.float64, delta=1e-6, device=False):
+    """Returns (outputs, analytic gradient, numerical gradient) of one op logic, the
+    gradients concatenated over the operands."""
+    logic_id, sizes, n_const, n_out = LOGICS[name]
+    flat = np.concatenate([np.asarray(o, np.float64).ravel() for o in operands] + [np.asarray(constants, np.float64).ravel()])
+    assert flat.size == sum(sizes) + n_const, (name, flat.size)
+    up = np.ones(n_out) if upstream is None else np.asarray(upstream, np.float64)
+    out = np.zeros(64, np.float64)
+    n = load().xad_test_eval_logic(ctypes.c_int(1 if device else 0), ctypes.c_int(logic_id),
+                                   ctypes.c_int(1 if np.dtype(dtype) == np.float64 else 0),
+                                   flat.ctypes.data_as(ctypes.c_void_p), ctypes.c_int(flat.size), up.ctypes.data_as(ctypes.c_void_p),
+                                   ctypes.c_int(up.size), ctypes.c_double(delta), out.ctypes.data_as(ctypes.c_void_p))
+    n_in = sum(sizes)
+    assert n == n_out + 2 * n_in, (name, n)
+    return out[:n_out].copy(), out[n_out:n_out + n_in].copy(), out[n_out + n_in:n].copy()
+
+
+def parallel_accumulation(threads, block):
+    out = np.zeros(3, np.float64)
+    rc = load().xad_test_parallel_accumulation(ctypes.c_size_t(threads), ctypes.c_int(block), out.ctypes.data_as(ctypes.c_void_p))
+    assert rc == 0
+    return out
+
+
+def shared_accumulation(blocks, threads):
+    out = np.zeros(2 * blocks, np.float64)
+    rc = load().xad_test_shared_accumulation(ctypes.c_int(blocks), ctypes.c_int(threads), out.ctypes.data_as(ctypes.c_void_p))
+    assert rc == 0
+    return out.reshape(blocks, 2)

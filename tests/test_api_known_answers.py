@@ -1,0 +1,82 @@
+"""Known answers for the public operator API, on the host cores and on the GPU.
+
+The cases are in tests/native/api_cases.cuh, each a restatement of a test of the
+reference (file and lines cited there); the numbers below are the ones those
+tests expect.  The same compiled case functions run on both sides.
+"""
+import math
+
+import numpy as np
+import pytest
+
+from tests import _native
+
+E = math.e
+
+EXPECTED = {
+    0: [1, 2, 3, 0, 2, 4, 0, 0, 0],
+    1: [10, 11, 12, 0, 3, 6, 3.5, 7.5, 7.5, 1.25, -2.5, 0],
+    2: [1, 2, 3, 4, 5, 6, 1, 4, 2, 5, 3, 6, 2.5, 0],
+    3: [19, 22, 43, 50, 17, 23, 39, 53],
+    4: [1, 0, 0, 0, 2, 0, 0, 0, 3] + [1, 2, 6, 8, 15, 18] + [1, 4, 9, 4, 10, 18] + [2, 4, 0, 3],
+    5: [1, 2, 2, 4, 3, 6, 2, 5] + [1, 2, 2, 4, 5, 5] + [1, 2, 3, 4, 5, 6] + [6, 10] + [1, 2, 3],
+    6: [5, 7, 9, 3, 3, 3, 4, 10, 18, 4, 2.5, 2] + [4, 6, 8] + [4, 4, 4] + [2, 3, 4] + [-2, -3, -4] + [14, 18],
+    7: [3.5, 4.5, 5.5, 1, 1, 1] + [0.5, 1.5, 2.5, 1, 1, 1] + [1.5, 3, 4.5, 1.5, 1.5, 1.5] + [1 / 3, 2 / 3, 1, 1 / 3, 1 / 3, 1 / 3],
+    8: [6, -2.5, 1, 1] + [-2, -3.5, 1, -1] + [8, -1.5, 4, 0.5, 2, -3] + [0.5, -6, 0.25, 2, -0.125, 12],
+    9: [3.5] * 4 + [10] + [3, 5, 7] + [3] + [1, 1, 1] + [1.5, 6],
+    10: [6, 4] + [9, 4] + [12, 7] + [-1.2, 2, 2] + [12, 8, 6, 16],
+    11: [2.5, 1.5, 0.75, 1.125, 1.5, 0.75, 1.125],
+    12: [4.625, 2.5, -3.5] + [2 * (E + E ** -2), 2 * E, 2 * E ** -2],
+}
+
+
+def _math_expectations():
+    x = 1.0
+    sig = lambda v: 1 / (1 + math.exp(-v))
+    gelu = 0.5 * x * (1 + math.tanh(0.7978845608028654 * (x + 0.044715 * x ** 3)))
+    return [math.exp(x), 1.0, math.sin(x), math.cos(x), math.tan(x), math.sinh(x), math.cosh(x), math.tanh(x), 2.0, 8.0,
+            2.5, 2.0, 1.0, 0.5, 0.0, 2.0, -0.01, math.exp(-1) - 1, math.log(2), sig(1.0), gelu, math.sin(2.5), math.cos(2.5)]
+
+
+def _check(case_id, got):
+    if case_id in (13, 14):
+        want = _math_expectations()
+        tol = 1e-6 if case_id == 13 else 1e-12  # fp32: tests/test_math_dispatcher.cu uses 1e-5; fp64: 1e-10
+    else:
+        want = EXPECTED[case_id]
+        tol = 1e-6
+    assert len(got) == len(want), (case_id, len(got), len(want))
+    assert np.allclose(got, want, rtol=tol, atol=tol), (case_id, list(got), want)
+
+
+@pytest.mark.parametrize("case_id", sorted(EXPECTED) + [13, 14])
+def test_case_on_host(case_id):
+    _check(case_id, _native.run_case(case_id, device=False))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("case_id", sorted(EXPECTED) + [13, 14])
+def test_case_on_gpu(gpu, case_id):
+    got = _native.run_case(case_id, device=True)
+    _check(case_id, got)
+    host = _native.run_case(case_id, device=False)
+    tol = 2e-6 if case_id == 13 else 1e-12
+    assert np.allclose(got, host, rtol=tol, atol=tol)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("threads,block", [(10_000, 256), (100_000, 512)])
+def test_concurrent_add_grad_on_global_memory(gpu, threads, block):
+    """tests/test_parallel_gradient_accumulation.cu:94-110 and :162-167 of the reference."""
+    got = _native.parallel_accumulation(threads, block)
+    assert got[0] == threads and got[1] == threads
+    want = 3.0 * threads + 0.002 * (threads - 1) * threads / 2
+    assert abs(got[2] - want) <= 1e-6 * want
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("blocks,threads", [(1, 128), (4, 64)])
+def test_concurrent_add_grad_on_lds(gpu, blocks, threads):
+    """tests/test_shared_memory_atomic.cu:102-109 and :179-187 of the reference."""
+    got = _native.shared_accumulation(blocks, threads)
+    assert np.all(got[:, 0] == threads) and np.all(got[:, 1] == 2 * threads)

@@ -1,0 +1,112 @@
+"""Pins the oracle's per-op forward and backward rules (oracle/oracle_ops.inc).
+
+Each rule is a restatement of one op-logic struct of the reference.  Before the
+library is checked against them they are pinned by:
+  - the forward values of independent numpy formulas,
+  - central finite differences, in fp64, of the oracle's own forward (with a
+    random upstream gradient, so a wrong sign, a dropped term or two swapped
+    outputs changes the result),
+  - textbook identities (a matrix times its inverse, orthonormal rotations).
+"""
+import zlib
+
+import numpy as np
+import pytest
+
+from tests import _native, _oracle_ops
+from tests._metrics import abs_or_rel
+
+NAMES = sorted(_native.LOGICS)
+
+
+def _numpy_forward(name, ops, k):
+    a = ops[0]
+    b = ops[1] if len(ops) > 1 else None
+    if name == "exp": return np.exp(a)
+    if name == "sin": return np.sin(a)
+    if name == "cos": return np.cos(a)
+    if name == "sigmoid": return 1 / (1 + np.exp(-a))
+    if name == "neg": return -a
+    if name == "squared": return a * a
+    if name == "sum": return np.array([a.sum()])
+    if name == "l1_norm": return np.array([np.abs(a).sum()])
+    if name == "l2_norm": return np.array([np.sqrt((a * a).sum())])
+    if name == "add_constant": return a + k[0]
+    if name == "sub_constant": return a - k[0]
+    if name == "mul_constant": return a * k[0]
+    if name == "div_constant": return a / k[0]
+    if name == "const_add": return a + k
+    if name == "const_sub": return a - k
+    if name == "sym_matrix2_inv":
+        inv = np.linalg.inv(np.array([[a[0], a[1]], [a[1], a[2]]]))
+        return np.array([inv[0, 0], inv[0, 1], inv[1, 1]])
+    if name == "quaternion_to_rotation_matrix":
+        x, y, z, w = a
+        return np.array([1 - 2 * (y * y + z * z), 2 * (x * y - z * w), 2 * (x * z + y * w), 2 * (x * y + z * w), 1 - 2 * (x * x + z * z),
+                         2 * (y * z - x * w), 2 * (x * z - y * w), 2 * (y * z + x * w), 1 - 2 * (x * x + y * y)])
+    if name == "broadcast_logic": return np.full(4, a[0])
+    if name == "add": return a + b
+    if name == "sub": return a - b
+    if name == "mul": return a * b
+    if name == "div": return a / b
+    if name == "matmul_2x2": return (a.reshape(2, 2) @ b.reshape(2, 2)).ravel()
+    if name == "matmul_3x3": return (a.reshape(3, 3) @ b.reshape(3, 3)).ravel()
+    if name == "matvec_2x3": return a.reshape(2, 3) @ b
+    if name == "vecmat_3x2": return a @ b.reshape(3, 2)
+    R = lambda t: np.array([[np.cos(t), -np.sin(t)], [np.sin(t), np.cos(t)]])
+    if name == "generate_covariance_matrix": return (R(b[0]) @ np.diag(a)).ravel()
+    if name == "matrix_to_covariance_3param":
+        S = a.reshape(2, 2) @ a.reshape(2, 2).T
+        return np.array([S[0, 0], S[0, 1], S[1, 1]])
+    if name == "scale_rotation_to_covariance_3param":
+        M = R(b[0]) @ np.diag(a)
+        S = M @ M.T
+        return np.array([S[0, 0], S[0, 1], S[1, 1]])
+    if name == "mahalanobis_distance":
+        A = np.array([[b[0], b[1]], [b[1], b[2]]])
+        return np.array([a @ A @ a])
+    if name == "mahalanobis_distance_with_center":
+        A = np.array([[b[0], b[1]], [b[1], b[2]]])
+        d = k - a
+        return np.array([d @ A @ d])
+    raise KeyError(name)
+
+
+@pytest.mark.parametrize("name", NAMES)
+def test_forward_matches_numpy_and_backward_matches_finite_differences(oracle, name):
+    rng = np.random.default_rng(zlib.crc32(name.encode()))
+    _, sizes, _, n_out = _native.LOGICS[name]
+    for _ in range(25):
+        ops, k = _oracle_ops.sample_inputs(name, rng)
+        up = rng.uniform(-1.5, 1.5, n_out)
+        y, g = _oracle_ops.evaluate(oracle, name, ops, k, up, np.float64)
+        assert np.allclose(y, _numpy_forward(name, ops, k), rtol=1e-12, atol=1e-12), name
+        flat = np.concatenate(ops)
+        h = 1e-6
+        fd = np.zeros_like(flat)
+        for i in range(flat.size):
+            hi, lo = flat.copy(), flat.copy()
+            hi[i] += h
+            lo[i] -= h
+            split = lambda v: [v[sum(sizes[:j]):sum(sizes[:j + 1])] for j in range(len(sizes))]
+            fd[i] = (up @ (_numpy_forward(name, split(hi), k) - _numpy_forward(name, split(lo), k))) / (2 * h)
+        assert abs_or_rel(g, fd).max() < 1e-6, (name, g, fd)
+
+
+def test_quirks_of_the_reference_rules(oracle):
+    # determinant guard of the 2x2 inverse: |det| < 1e-8 is replaced by +1e-8 (both passes)
+    y, g = _oracle_ops.evaluate(oracle, "sym_matrix2_inv", [np.array([1.0, 1.0, 1.0])])
+    assert np.allclose(y, [1e8, -1e8, 1e8])
+    assert np.isfinite(g).all()
+    # L1: sign(0) = 0;  L2: no gradient at (numerically) zero norm
+    _, g = _oracle_ops.evaluate(oracle, "l1_norm", [np.array([0.0, 2.0, -3.0, 0.0])])
+    assert np.array_equal(g, [0.0, 1.0, -1.0, 0.0])
+    _, g = _oracle_ops.evaluate(oracle, "l2_norm", [np.zeros(4)])
+    assert np.array_equal(g, np.zeros(4))
+    # identities: inverse of the covariance of a rotation by theta with scales s
+    S, _ = _oracle_ops.evaluate(oracle, "scale_rotation_to_covariance_3param", [np.array([1.5, 0.4]), np.array([0.7])])
+    inv, _ = _oracle_ops.evaluate(oracle, "sym_matrix2_inv", [S])
+    prod = np.array([[S[0], S[1]], [S[1], S[2]]]) @ np.array([[inv[0], inv[1]], [inv[1], inv[2]]])
+    assert np.allclose(prod, np.eye(2), atol=1e-12)
+    Rm, _ = _oracle_ops.evaluate(oracle, "quaternion_to_rotation_matrix", [np.array([0.5, 0.5, 0.5, 0.5])])
+    assert np.allclose(Rm.reshape(3, 3) @ Rm.reshape(3, 3).T, np.eye(3), atol=1e-12)
