@@ -85,7 +85,8 @@ def accumulate_report(ins, seed, with_oracle):
     n = min(ins[0].numel(), 16 * 1024 * 1024)
     sub = [t[:n] for t in ins]
     host = [t.cpu().numpy() for t in sub] if with_oracle else None
-    out = {"n": n, "bytes_per_thread": accumulate.BYTES_PER_THREAD, "slots": {}}
+    out = {"n": n, "bytes_per_thread": accumulate.BYTES_PER_THREAD, "slots": {},
+           "lds_atomic_cycles_per_wavefront_instruction": accumulate.lds_atomic_cycles()}
     for num_slots in (64, 4096, 262144):
         slot = torch.empty(n, dtype=torch.int32, device=dev)
         accumulate.zipf_(slot, seed, 10, num_slots, 1.1)
@@ -202,8 +203,10 @@ def main():
     ap.add_argument("--n", type=int, default=N_FULL, help="problems per step (default: the full 64 Mi)")
     ap.add_argument("--seed", type=int, default=1234)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs (profiling runs)")
-    ap.add_argument("--counter-probe", action="store_true",
-                    help="launch only a 256 Mi-float copy and three chain passes, then exit (for rocprofv3 --pmc runs)")
+    ap.add_argument("--counter-probe", choices=("chain", "accumulate", "splat"), default=None,
+                    help="launch a few kernels of one leg and exit, for rocprofv3 --pmc runs: chain = a 256 Mi-float "
+                         "copy then three chain passes; accumulate = naive and staged accumulation at 64 and 4096 slots; "
+                         "splat = two iterations of the 200k-Gaussian step")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (got --gpus %d)" % args.gpus)
@@ -221,13 +224,40 @@ def main():
     rng.chain_inputs_(ins, args.seed)
     torch.cuda.synchronize()
 
-    if args.counter_probe:
+    if args.counter_probe == "chain":
         # known traffic first (1 GiB read + 1 GiB written), then the kernel under study
         chain.stream_copy(torch.cat(ins[:4]), torch.cat(outs[:4]))
         for _ in range(3):
             chain.forward_backward(ins, outs)
         torch.cuda.synchronize()
-        print(json.dumps({"counter_probe": True, "n": n, "copy_floats": 4 * n}))
+        print(json.dumps({"counter_probe": "chain", "n": n, "copy_floats": 4 * n}))
+        return
+    if args.counter_probe == "accumulate":
+        from xyz_autodiff_cuda_amd import accumulate
+
+        m = 16 * 1024 * 1024
+        sub = [t[:m] for t in ins]
+        for num_slots in (64, 4096):
+            slot = torch.empty(m, dtype=torch.int32, device=dev)
+            accumulate.zipf_(slot, args.seed, 10, num_slots, 1.1)
+            grads = torch.zeros(num_slots, 6, dtype=torch.float32, device=dev)
+            for name in ("global_atomics", "auto", "wave_lds"):
+                accumulate.accumulate_chain_gradients(sub, slot, grads, name)
+        torch.cuda.synchronize()
+        print(json.dumps({"counter_probe": "accumulate", "n": m, "order": "per slots in (64, 4096): global_atomics, auto, wave_lds"}))
+        return
+    if args.counter_probe == "splat":
+        from xyz_autodiff_cuda_amd import splat
+
+        del ins, outs
+        G, W, H, scale = 200_000, 2048, 2048, (0.5, 40.0)
+        target = splat.synthetic_target(G, W, H, seed=77, scale_px=scale, noise=0.02)
+        params, depth = splat.synthetic_scene(G, W, H, seed=args.seed, scale_px=scale)
+        ctx = splat.SplatContext(W, H, G, pair_capacity_hint=9_000_000)
+        for _ in range(2):
+            ctx.step(params, depth, target, want_loss=False)
+        torch.cuda.synchronize()
+        print(json.dumps({"counter_probe": "splat", "pairs": ctx.stats()["pairs"]}))
         return
 
     for _ in range(args.warmup):

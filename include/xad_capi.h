@@ -192,6 +192,17 @@ int xad_adam_step_f32(size_t n, int rows, float* params, const float* grads, flo
                       int iteration, void* stream);
 
 /* ---------------------------------------------------------------------------
+ * Hardware probe behind the accumulator's design: shader cycles the LDS pipeline
+ * of a CU spends on one wavefront-wide atomic add (16 wavefronts of one block
+ * issuing back to back), by element type (0 float, 1 double, 2 uint32, 3 uint64)
+ * and address pattern (0 sixty-four distinct addresses, 1 one address, 2 sixteen
+ * lanes on one address, 3 eight lanes per address, 4 stride of six elements).
+ * Synchronous; allocates and frees small device buffers.  No counterpart in the
+ * reference.
+ */
+int xad_probe_lds_atomic_cycles(int element, int pattern, double* cycles_per_instruction);
+
+/* ---------------------------------------------------------------------------
  * Synthetic inputs: counter-based generator, element i of a fill is a pure
  * function of (seed, stream_id, i).  The reference seeds std::mt19937 on the
  * host and uploads (examples/mini-gaussian-splatting/gaussian_parameters.cu:27-66);

@@ -45,6 +45,7 @@ SIGNATURES = {
     "xad_splat_set_profiling": [_vp, _int],
     "xad_splat_get_stats": [_vp, ctypes.POINTER(_u64), ctypes.POINTER(ctypes.c_uint32), ctypes.POINTER(_flt)],
     "xad_adam_step_f32": [_sz, _int, _vp, _vp, _vp, _vp, ctypes.POINTER(_flt), _flt, _flt, _flt, _int, _vp],
+    "xad_probe_lds_atomic_cycles": [_int, _int, ctypes.POINTER(ctypes.c_double)],
     "xad_rng_zipf_i32": [_vp, _sz, _u64, _u64, _int, ctypes.c_double, _vp],
     "xad_rng_uniform_f32": [_vp, _sz, _u64, _u64, _flt, _flt, _vp],
     "xad_rng_normal_f32": [_vp, _sz, _u64, _u64, _flt, _flt, _vp],
