@@ -118,6 +118,57 @@ def accumulate_report(ins, seed, with_oracle):
     return out
 
 
+def linreg_report(with_oracle):
+    """Least-squares example (fp64, four parameters shared by all samples): gradient
+    sums over 16 Mi samples per strategy, and the reference's training run (100 000
+    samples, batch 8192, 10 000 steps) entirely on the device."""
+    import time
+
+    import numpy as np
+    import torch
+
+    from xyz_autodiff_cuda_amd import linreg
+
+    dev = torch.device("cuda:0")
+    n = 16 * 1024 * 1024
+    x1, x2, y = (torch.from_numpy(a).to(dev) for a in linreg.synthetic_data(n, seed=1))
+    params = torch.tensor([0.4, 1.3, -0.2, 0.1], dtype=torch.float64, device=dev)
+    out = {"n": n, "bytes_per_sample": linreg.BYTES_PER_SAMPLE, "gradient": {}}
+    want = None
+    if with_oracle:
+        from tests import _oracle
+
+        t0 = time.perf_counter()
+        want = _oracle.load().linreg_gradient(x1.cpu().numpy(), x2.cpu().numpy(), y.cpu().numpy(), params.cpu().numpy())
+        out["cpu_oracle_ms"] = (time.perf_counter() - t0) * 1e3
+    for name, reps in (("wave_lds", 10), ("lds_leaves", 3), ("global_atomics", 1)):
+        times = []
+        for _ in range(reps + 1):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            got = linreg.batch_gradient(x1, x2, y, params, strategy=name)
+            b.record()
+            torch.cuda.synchronize()
+            times.append(a.elapsed_time(b))
+        ms = sorted(times[1:])[len(times[1:]) // 2]
+        item = {"ms": ms, "GBps": linreg.BYTES_PER_SAMPLE * n / ms / 1e6}
+        if want is not None:
+            item["max_rel_err"] = float(np.max(np.abs(got.cpu().numpy() - want) / np.abs(want)))
+        out["gradient"][name] = item
+    out["gradient"]["speedup_vs_global_atomics"] = out["gradient"]["global_atomics"]["ms"] / out["gradient"]["wave_lds"]["ms"]
+
+    total, batch, epochs = 100_000, 8192, 10_000
+    sx1, sx2, sy = (torch.from_numpy(a).to(dev) for a in linreg.synthetic_data(total, seed=0))
+    p = torch.tensor(linreg.INITIAL_PARAMS, dtype=torch.float64, device=dev)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    linreg.sgd(sx1, sx2, sy, p, batch, epochs, seed=1)
+    dt = time.perf_counter() - t0
+    out["sgd"] = {"samples": total, "batch": batch, "steps": epochs, "seconds": dt, "steps_per_s": epochs / dt,
+                  "final_params": p.cpu().tolist(), "true_params": list(linreg.TRUE_PARAMS)}
+    return out
+
+
 def splat_report(with_oracle, iters=30):
     """Configs 4 and 5: one training iteration = forward + backward + Adam (lr 1e-2).
     Reports iterations/s, the per-kernel time split, pair statistics, and the CPU
@@ -335,6 +386,7 @@ def main():
     del ins, outs
     torch.cuda.empty_cache()
     record["splat"] = splat_report(with_oracle=not args.no_cpu)
+    record["linreg"] = linreg_report(with_oracle=not args.no_cpu)
     print(json.dumps(record))
 
 

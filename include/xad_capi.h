@@ -40,6 +40,11 @@ const char* xad_last_error(void);
 /* ABI revision of this library; bumped on incompatible changes. */
 int xad_abi_version(void);
 
+/* SHA-256 (hex) of the sources this library was built from, as computed by its
+ * build script; "" for a build that did not record it.  Lets a loader refuse a
+ * library that is older than the sources next to it. */
+const char* xad_source_digest(void);
+
 /* ---------------------------------------------------------------------------
  * Per-thread forward + backward of the benchmark graph, structure of arrays.
  *
@@ -190,6 +195,56 @@ int xad_splat_get_stats(const xad_splat_context* ctx, uint64_t* pairs, uint32_t*
 int xad_adam_step_f32(size_t n, int rows, float* params, const float* grads, float* m, float* v,
                       const float* row_learning_rates, float beta1, float beta2, float eps,
                       int iteration, void* stream);
+
+/* ---------------------------------------------------------------------------
+ * Least-squares fit of  y ~ (x1 - a)^2 + b (x2 - c)^2 + d  by mini-batch SGD, fp64:
+ * four parameters shared by every sample, the extreme-contention case of
+ * gradient accumulation.
+ *
+ * Stands in for the kernels of examples/optimization/linear_regression_sgd.cu:
+ * select_batch_kernel (:68-81), parallel_gradient_computation_kernel (:86-123),
+ * update_parameters_kernel (:126-134) and the loop of main (:186-229).  The
+ * per-sample graph is the one of
+ * examples/optimization/tests/test_linear_regression_gradient.cu:47-78, i.e. the
+ * squared residual (the example itself differentiates the un-squared node,
+ * :119-122, on a batch of one, :204-208).  Samples are three arrays, not an
+ * array of {x1, x2, y} structs.
+ *
+ *   strategy  how the four gradients of all samples are summed:
+ *     GLOBAL_ATOMICS  VariableRef leaves on the global gradient, one fp64 atomic
+ *                     per sample and parameter (the reference pattern)
+ *     LDS_LEAVES      the same graph with accumulator leaves (per-block LDS
+ *                     table, one global atomic per block and element)
+ *     WAVE_LDS        register leaves, per-lane running sums, wavefront
+ *                     reduction, then the LDS table
+ *   x1, x2, y   device, `total` doubles each
+ *   rows        device, n sample indices into x1/x2/y, or NULL for samples 0..n-1
+ *   params      device, 4 doubles: a, b, c, d
+ *   out         device, 5 doubles, overwritten: sum over the n samples of
+ *               d loss / d (a, b, c, d) and of loss = (prediction - y)^2
+ */
+#define XAD_LINREG_GLOBAL_ATOMICS 0
+#define XAD_LINREG_LDS_LEAVES 1
+#define XAD_LINREG_WAVE_LDS 2
+int xad_linreg_gradient_f64(int strategy, size_t n, size_t total,
+                            const double* x1, const double* x2, const double* y, const int* rows,
+                            const double* params, double* out, void* stream);
+/* `epochs` SGD steps, entirely on the device: step e draws `batch` rows with
+ * replacement, row of draw i = random bits (seed, stream 0, e * batch + i)
+ * modulo total (see xad_host_rng_bits), sums the gradients with WAVE_LDS, and
+ * updates  p -= lr(e) * sum / batch  with  lr(e) = lr_first * (lr_last /
+ * lr_first)^(e / epochs)  (linear_regression_sgd.cu:137-140).  params (device, 4
+ * doubles) is updated in place; loss_history (device, `epochs` doubles, or NULL)
+ * receives the mean batch loss before each update.  Synchronous: returns when
+ * the last step has finished. */
+int xad_linreg_sgd_f64(size_t total, const double* x1, const double* x2, const double* y,
+                       double* params, int batch, int epochs, double lr_first, double lr_last,
+                       uint64_t seed, double* loss_history, void* stream);
+/* Host cores: the same graph templates compiled for the CPU, one thread; all
+ * pointers host. */
+int xad_host_linreg_gradient_f64(size_t n, size_t total,
+                                 const double* x1, const double* x2, const double* y, const int* rows,
+                                 const double* params, double* out);
 
 /* ---------------------------------------------------------------------------
  * Hardware probe behind the accumulator's design: shader cycles the LDS pipeline

@@ -77,10 +77,27 @@ __device__ __forceinline__ float read_lane(float v, int lane) {
     return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
 }
 
+// 64-bit values travel as two 32-bit halves.
+template <int Ctrl>
+__device__ __forceinline__ double dpp_add(double v) {
+    const std::uint64_t u = __builtin_bit_cast(std::uint64_t, v);
+    const unsigned lo = __builtin_amdgcn_update_dpp(0, static_cast<int>(u), Ctrl, 0xF, 0xF, true);
+    const unsigned hi = __builtin_amdgcn_update_dpp(0, static_cast<int>(u >> 32), Ctrl, 0xF, 0xF, true);
+    return v + __builtin_bit_cast(double, (static_cast<std::uint64_t>(hi) << 32) | lo);
+}
+
+__device__ __forceinline__ double read_lane(double v, int lane) {
+    const std::uint64_t u = __builtin_bit_cast(std::uint64_t, v);
+    const unsigned lo = __builtin_amdgcn_readlane(static_cast<int>(u), lane);
+    const unsigned hi = __builtin_amdgcn_readlane(static_cast<int>(u >> 32), lane);
+    return __builtin_bit_cast(double, (static_cast<std::uint64_t>(hi) << 32) | lo);
+}
+
 // Sum of v over all 64 lanes, returned to every lane.  Four DPP steps reduce
 // each row of 16 (quad swaps, then the two mirrors), four scalar reads combine
 // the rows.
-__device__ __forceinline__ float sum(float v) {
+template <typename V>
+__device__ __forceinline__ V sum(V v) {
     v = dpp_add<0xB1>(v);   // quad_perm [1,0,3,2]
     v = dpp_add<0x4E>(v);   // quad_perm [2,3,0,1]
     v = dpp_add<0x141>(v);  // row_half_mirror
@@ -93,7 +110,6 @@ __device__ __forceinline__ float sum(float v) {
 template <typename T, int Width, Strategy S = Strategy::LdsAtomics, int PeelRounds = 8, int MinGroup = 4,
           typename TableT = double>
 class BlockAccumulator {
-    static_assert(sizeof(T) == 4 || S != Strategy::WaveThenLds, "the wavefront level is implemented for 4-byte values");
 
 public:
     using table_type = TableT;

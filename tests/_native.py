@@ -29,7 +29,16 @@ def load():
     if _lib is None:
         if not os.path.exists(LIB_PATH):
             raise ImportError("tests/native/libxad_api_tier.so is not built; run `python tests/native/build.py`")
-        _lib = ctypes.CDLL(LIB_PATH)
+        lib = ctypes.CDLL(LIB_PATH)
+        lib.xad_test_source_digest.restype = ctypes.c_char_p
+        import importlib.util
+
+        spec = importlib.util.spec_from_file_location("xad_native_build", os.path.join(HERE, "native", "build.py"))
+        build = importlib.util.module_from_spec(spec)
+        spec.loader.exec_module(build)
+        if lib.xad_test_source_digest().decode() != build.source_digest():
+            raise ImportError("tests/native/libxad_api_tier.so is older than its sources; run `python tests/native/build.py`")
+        _lib = lib
     return _lib
 
 

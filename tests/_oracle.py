@@ -136,3 +136,32 @@ class Oracle:
         P = ctypes.c_void_p
         fn(ctypes.c_long(p.size), p.ctypes.data_as(P), g.ctypes.data_as(P), m.ctypes.data_as(P), v.ctypes.data_as(P),
            ctypes.c_float(lr), ctypes.c_float(beta1), ctypes.c_float(beta2), ctypes.c_float(eps), ctypes.c_int(iteration))
+
+    def linreg_gradient(self, x1, x2, y, params, rows=None):
+        """-> array of 5: gradient sums for (a, b, c, d) and the loss sum."""
+        x1, x2, y, params = (np.ascontiguousarray(a, dtype=np.float64) for a in (x1, x2, y, params))
+        if rows is not None:
+            rows = np.ascontiguousarray(rows, dtype=np.int32)
+        n = rows.size if rows is not None else x1.size
+        out = np.zeros(5, np.float64)
+        fn = self.lib.oracle_linreg_gradient_f64
+        fn.restype = None
+        P = ctypes.c_void_p
+        fn(ctypes.c_long(n), x1.ctypes.data_as(P), x2.ctypes.data_as(P), y.ctypes.data_as(P),
+           rows.ctypes.data_as(P) if rows is not None else P(0), params.ctypes.data_as(P), out.ctypes.data_as(P))
+        return out
+
+    def linreg_sgd(self, x1, x2, y, rows, params, batch, epochs, lr_first, lr_last):
+        """rows: int32 (epochs * batch).  -> (final params, loss history)."""
+        x1, x2, y = (np.ascontiguousarray(a, dtype=np.float64) for a in (x1, x2, y))
+        rows = np.ascontiguousarray(rows, dtype=np.int32)
+        assert rows.size == batch * epochs
+        p = np.array(params, dtype=np.float64)
+        history = np.zeros(epochs, np.float64)
+        fn = self.lib.oracle_linreg_sgd_f64
+        fn.restype = None
+        P = ctypes.c_void_p
+        fn(x1.ctypes.data_as(P), x2.ctypes.data_as(P), y.ctypes.data_as(P), rows.ctypes.data_as(P), p.ctypes.data_as(P),
+           ctypes.c_int(batch), ctypes.c_int(epochs), ctypes.c_double(lr_first), ctypes.c_double(lr_last),
+           history.ctypes.data_as(P))
+        return p, history

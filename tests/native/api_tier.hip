@@ -144,6 +144,11 @@ bool ok(hipError_t e) { return e == hipSuccess; }
 
 }  // namespace
 
+#ifndef XAD_TEST_SOURCE_DIGEST
+#define XAD_TEST_SOURCE_DIGEST ""
+#endif
+extern "C" const char* xad_test_source_digest(void) { return XAD_TEST_SOURCE_DIGEST; }
+
 extern "C" int xad_test_case_capacity(void) { return xad_test::kCaseCapacity; }
 
 extern "C" int xad_test_run_case_host(int id, double* out) { return xad_test::run_case(id, out); }

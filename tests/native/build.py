@@ -1,4 +1,5 @@
 """Builds tests/native/libxad_api_tier.so (the API test tier) for gfx950 + host."""
+import hashlib
 import os
 import subprocess
 
@@ -7,12 +8,26 @@ ROOT = os.path.dirname(os.path.dirname(HERE))
 LIB = os.path.join(HERE, "libxad_api_tier.so")
 
 
+def source_digest():
+    """SHA-256 over this directory's sources and the library headers they include."""
+    h = hashlib.sha256()
+    files = [os.path.join(HERE, f) for f in os.listdir(HERE) if f.endswith((".hip", ".cuh"))]
+    for dirpath, _, names in os.walk(os.path.join(ROOT, "include")):
+        files += [os.path.join(dirpath, f) for f in names if f.endswith((".cuh", ".h"))]
+    for path in sorted(files):
+        h.update(os.path.relpath(path, ROOT).encode() + b"\0")
+        with open(path, "rb") as f:
+            h.update(f.read() + b"\0")
+    return h.hexdigest()
+
+
 def build():
     cmd = [
         os.environ.get("HIPCC", "/opt/rocm/bin/hipcc"), "--offload-arch=gfx950", "-std=c++20", "-O2", "-fPIC", "-shared",
         "-fno-gpu-sanitize", "-march=x86-64-v3", "-munsafe-fp-atomics",
         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-command-line-argument",
         "-I" + os.path.join(ROOT, "include"), "-I" + os.path.join(ROOT, "include", "mini-gaussian-splatting"),
+        "-DXAD_TEST_SOURCE_DIGEST=\"%s\"" % source_digest(),
         os.path.join(HERE, "api_tier.hip"), "-o", LIB,
     ]
     proc = subprocess.run(cmd, capture_output=True, text=True)

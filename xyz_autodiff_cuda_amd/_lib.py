@@ -32,6 +32,7 @@ _flt = ctypes.c_float
 SIGNATURES = {
     "xad_last_error": [],
     "xad_abi_version": [],
+    "xad_source_digest": [],
     "xad_chain_forward_backward_f32": [_sz] + [_vp] * 13 + [_vp],
     "xad_chain_forward_backward_f32_layout": [_sz] + [_vp] * 13 + [_int, _vp],
     "xad_stream_copy_f32": [_sz, _vp, _vp, _vp],
@@ -45,6 +46,9 @@ SIGNATURES = {
     "xad_splat_set_profiling": [_vp, _int],
     "xad_splat_get_stats": [_vp, ctypes.POINTER(_u64), ctypes.POINTER(ctypes.c_uint32), ctypes.POINTER(_flt)],
     "xad_adam_step_f32": [_sz, _int, _vp, _vp, _vp, _vp, ctypes.POINTER(_flt), _flt, _flt, _flt, _int, _vp],
+    "xad_linreg_gradient_f64": [_int, _sz, _sz, _vp, _vp, _vp, _vp, _vp, _vp, _vp],
+    "xad_linreg_sgd_f64": [_sz, _vp, _vp, _vp, _vp, _int, _int, ctypes.c_double, ctypes.c_double, _u64, _vp, _vp],
+    "xad_host_linreg_gradient_f64": [_sz, _sz, _vp, _vp, _vp, _vp, _vp, _vp],
     "xad_probe_lds_atomic_cycles": [_int, _int, ctypes.POINTER(ctypes.c_double)],
     "xad_rng_zipf_i32": [_vp, _sz, _u64, _u64, _int, ctypes.c_double, _vp],
     "xad_rng_uniform_f32": [_vp, _sz, _u64, _u64, _flt, _flt, _vp],
@@ -52,7 +56,7 @@ SIGNATURES = {
     "xad_host_rng_bits": [_vp, _sz, _u64, _u64, _u64],
     "xad_host_rng_uniform_f32": [_vp, _sz, _u64, _u64, _flt, _flt],
 }
-_RESTYPE = {"xad_last_error": ctypes.c_char_p, "xad_splat_destroy": None}
+_RESTYPE = {"xad_last_error": ctypes.c_char_p, "xad_source_digest": ctypes.c_char_p, "xad_splat_destroy": None}
 
 
 def load():
@@ -69,6 +73,14 @@ def load():
         fn = getattr(lib, name)
         fn.argtypes = argtypes
         fn.restype = _RESTYPE.get(name, ctypes.c_int)
+    from . import build
+
+    built_from = lib.xad_source_digest().decode()
+    if built_from != build.source_digest():
+        raise ImportError(
+            "libxad_hip.so was built from other sources than the ones next to it (digest %s...); "
+            "rebuild with `python -m xyz_autodiff_cuda_amd.build`" % built_from[:12]
+        )
     _lib = lib
     return lib
 

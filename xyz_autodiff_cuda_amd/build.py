@@ -6,6 +6,7 @@ hipcc cross-compiles without a GPU.  The host pass of the same translation
 units carries the host-core build of the templates (x86-64-v3: AVX2 + FMA, so
 the library runs on any recent host without depending on the build machine).
 """
+import hashlib
 import os
 import subprocess
 import sys
@@ -43,9 +44,27 @@ def sources():
     return sorted(os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".hip"))
 
 
-def _compile(src):
+def source_digest():
+    """SHA-256 over every file the library is built from (csrc/ and include/), by
+    relative path and content.  The build bakes it into the library
+    (xad_source_digest) so that a library older than its sources can be told."""
+    h = hashlib.sha256()
+    files = []
+    for base in (CSRC, os.path.join(ROOT, "include")):
+        for dirpath, _, names in os.walk(base):
+            files += [os.path.join(dirpath, f) for f in names if f.endswith((".hip", ".cuh", ".h"))]
+    for path in sorted(files):
+        h.update(os.path.relpath(path, ROOT).encode())
+        h.update(b"\0")
+        with open(path, "rb") as f:
+            h.update(f.read())
+        h.update(b"\0")
+    return h.hexdigest()
+
+
+def _compile(src, digest):
     obj = os.path.join(OBJ_DIR, os.path.basename(src) + ".o")
-    cmd = [HIPCC, *FLAGS, "-c", src, "-o", obj]
+    cmd = [HIPCC, *FLAGS, "-DXAD_SOURCE_DIGEST=\"%s\"" % digest, "-c", src, "-o", obj]
     proc = subprocess.run(cmd, capture_output=True, text=True)
     noise = "is not a recognized feature for this target"
     err = "\n".join(l for l in proc.stderr.splitlines() if noise not in l)
@@ -56,8 +75,9 @@ def _compile(src):
 
 def build(verbose=False):
     os.makedirs(OBJ_DIR, exist_ok=True)
+    digest = source_digest()
     with ThreadPoolExecutor(max_workers=min(8, os.cpu_count() or 1)) as pool:
-        results = list(pool.map(_compile, sources()))
+        results = list(pool.map(lambda src: _compile(src, digest), sources()))
     objs = [o for o, _ in results]
     if verbose:
         for _, err in results:

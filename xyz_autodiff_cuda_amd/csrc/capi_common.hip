@@ -10,3 +10,8 @@ char* last_error_buffer() {
 
 extern "C" const char* xad_last_error(void) { return xad::last_error_buffer(); }
 extern "C" int xad_abi_version(void) { return 1; }
+
+#ifndef XAD_SOURCE_DIGEST
+#define XAD_SOURCE_DIGEST ""
+#endif
+extern "C" const char* xad_source_digest(void) { return XAD_SOURCE_DIGEST; }
