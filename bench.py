@@ -118,6 +118,26 @@ def accumulate_report(ins, seed, with_oracle):
     return out
 
 
+def trainer_report():
+    """The trainer front-end at the size of config 5: iterations/s of xad_trainer_run (splatting
+    step + Adam per iteration, state resident on the device) on a synthetic target."""
+    import time
+
+    from xyz_autodiff_cuda_amd import splat, trainer
+
+    G, W, H = 200_000, 2048, 2048
+    target = splat.synthetic_target(G, W, H, seed=77, scale_px=(0.5, 40.0), noise=0.02).cpu().numpy()
+    config = trainer.TrainingConfig.defaults(num_gaussians=G, seed=1, target_image_path="synthetic")
+    t = trainer.Trainer(config, target)
+    first = t.run(5)
+    t0 = time.perf_counter()
+    last = t.run(50)
+    dt = time.perf_counter() - t0
+    t.close()
+    return {"gaussians": G, "image": [W, H], "iterations": 50, "iters_per_s": 50 / dt, "ms_per_iter": dt / 50 * 1e3,
+            "loss_after_5": first, "loss_after_55": last}
+
+
 def linreg_report(with_oracle):
     """Least-squares example (fp64, four parameters shared by all samples): gradient
     sums over 16 Mi samples per strategy, and the reference's training run (100 000
@@ -387,6 +407,7 @@ def main():
     torch.cuda.empty_cache()
     record["splat"] = splat_report(with_oracle=not args.no_cpu)
     record["linreg"] = linreg_report(with_oracle=not args.no_cpu)
+    record["trainer"] = trainer_report()
     print(json.dumps(record))
 
 

@@ -197,6 +197,96 @@ int xad_adam_step_f32(size_t n, int rows, float* params, const float* grads, flo
                       int iteration, void* stream);
 
 /* ---------------------------------------------------------------------------
+ * Splatting trainer front-end: configuration, image files, training loop,
+ * checkpoints.  Host-side counterpart of the reference's training program
+ * (examples/mini-gaussian-splatting/gaussian_splatting_training.cu,
+ * training_config.{h,cpp}, image_utils.{h,cpp}, GaussianCollection in
+ * gaussian_parameters.{h,cu}), around xad_splat_step and xad_adam_step_f32.
+ */
+
+/* The fields of TrainingConfig (training_config.h:7-31) with its defaults,
+ * followed by the additions of this build (seed, output directory, checkpoints). */
+typedef struct xad_training_config {
+    float lr_center, lr_scale, lr_rotation, lr_color, lr_opacity;
+    int max_iterations;   /* 500 */
+    int save_interval;    /* 25: an image every so many iterations */
+    int num_gaussians;    /* 1000 */
+    int save_images;      /* 1 */
+    float beta1, beta2, epsilon; /* 0.9, 0.999, 1e-8 */
+    char target_image_path[1024];
+    /* additions */
+    uint64_t seed;               /* 0: initial Gaussians are a function of the seed */
+    int checkpoint_interval;     /* 0 = only at the end (when checkpoint_path is set) */
+    char output_dir[1024];       /* "output" */
+    char checkpoint_path[1024];  /* "" = write none */
+    char resume_path[1024];      /* "" = start from random Gaussians */
+} xad_training_config;
+
+#define XAD_HELP_REQUESTED 4 /* returned by xad_training_config_parse for --help */
+
+void xad_training_config_defaults(xad_training_config* config);
+/* argv as given to main: <lr_center> <lr_scale> <lr_rotation> <lr_color>
+ * <lr_opacity> then --target PATH, --max-iterations N, --save-interval N,
+ * --num-gaussians N, --no-save-images, --beta1 V, --beta2 V, --epsilon V, --help
+ * (TrainingConfigParser::parse, training_config.cpp:29-88) and, added here,
+ * --seed N, --output-dir DIR, --checkpoint PATH, --checkpoint-interval N,
+ * --resume PATH.  Fails like the reference: fewer than five positional
+ * arguments "Insufficient arguments", an unknown option or an option without
+ * its value "Invalid argument", then the checks of validate_config
+ * (training_config.cpp:114-146) with its messages. */
+int xad_training_config_parse(int argc, const char* const* argv, xad_training_config* config);
+int xad_training_config_validate(const xad_training_config* config);
+/* The usage text (training_config.cpp:90-112). */
+const char* xad_training_usage(void);
+
+/* Image files: float RGB in [0, 1], height x width x 3, host memory.
+ * xad_image_load reads PNG (not interlaced) or binary PPM/PGM and allocates
+ * *rgb (release with xad_image_free); xad_image_save writes 8-bit PNG or PPM by
+ * the extension of `path`, quantising like save_image_jpeg (image_utils.cpp:39-56);
+ * xad_image_test_pattern fills the gradient of create_test_image (:58-77). */
+int xad_image_load(const char* path, int* width, int* height, float** rgb);
+void xad_image_free(float* rgb);
+int xad_image_save(const char* path, int width, int height, const float* rgb);
+int xad_image_test_pattern(int width, int height, float* rgb);
+
+/* A training run on the current device: parameters, gradients and Adam moments
+ * (9 rows x num_gaussians each, rows as in xad_splat_step), the target and the
+ * last rendering stay on the device.
+ *
+ * Initial Gaussians follow GaussianCollection::initialize_random
+ * (gaussian_parameters.cu:27-66): centre uniform over the image, log-scales
+ * max(1, U(0, 2)), rotation 0, colour U(0.1, 0.2), opacity logit U(0.05, 0.1),
+ * drawn from the counter-based generator with config->seed; depth (which the
+ * reference does not have) is U(0, 1) and is not trained.
+ * One iteration is the body of GaussianSplattingTrainer::train
+ * (gaussian_splatting_training.cu:127-160): gradients of the loss, then Adam
+ * with the five learning rates and iteration + 1 as the step count. */
+typedef struct xad_trainer xad_trainer;
+int xad_trainer_create(const xad_training_config* config, int width, int height,
+                       const float* target_rgb, xad_trainer** out);
+void xad_trainer_destroy(xad_trainer* trainer);
+/* Runs `iterations` iterations.  loss_out (host, may be NULL) receives the sum
+ * of squared errors of the last iteration's rendering, taken before its update. */
+int xad_trainer_run(xad_trainer* trainer, int iterations, double* loss_out);
+/* Iterations completed so far (continues from the checkpoint after a load). */
+int xad_trainer_iteration(const xad_trainer* trainer);
+/* The last rendering (zeros before the first iteration), to host memory. */
+int xad_trainer_download_image(xad_trainer* trainer, float* rgb);
+/* Copies of the state to host memory (9 x num_gaussians floats each, depth
+ * num_gaussians); any pointer may be NULL. */
+int xad_trainer_get_state(xad_trainer* trainer, float* params, float* m, float* v, float* depth);
+/* Replaces parameters and depth (host memory; NULL keeps the current ones). */
+int xad_trainer_set_params(xad_trainer* trainer, const float* params, const float* depth);
+/* Checkpoint = iteration count, image size, Gaussian count, learning rates and
+ * Adam constants, parameters, both Adam moments and depth, with a CRC-32 over
+ * the file.  Written to a temporary file and renamed.  Loading requires the
+ * same image size and Gaussian count and replaces iteration, parameters,
+ * moments and depth (the trainer's own configuration is kept).  The reference
+ * only mirrors its state to host memory (gaussian_parameters.cu:93-116). */
+int xad_trainer_save_checkpoint(xad_trainer* trainer, const char* path);
+int xad_trainer_load_checkpoint(xad_trainer* trainer, const char* path);
+
+/* ---------------------------------------------------------------------------
  * Least-squares fit of  y ~ (x1 - a)^2 + b (x2 - c)^2 + d  by mini-batch SGD, fp64:
  * four parameters shared by every sample, the extreme-contention case of
  * gradient accumulation.

@@ -46,6 +46,23 @@ SIGNATURES = {
     "xad_splat_set_profiling": [_vp, _int],
     "xad_splat_get_stats": [_vp, ctypes.POINTER(_u64), ctypes.POINTER(ctypes.c_uint32), ctypes.POINTER(_flt)],
     "xad_adam_step_f32": [_sz, _int, _vp, _vp, _vp, _vp, ctypes.POINTER(_flt), _flt, _flt, _flt, _int, _vp],
+    "xad_training_config_defaults": [_vp],
+    "xad_training_config_parse": [_int, ctypes.POINTER(ctypes.c_char_p), _vp],
+    "xad_training_config_validate": [_vp],
+    "xad_training_usage": [],
+    "xad_image_load": [ctypes.c_char_p, ctypes.POINTER(_int), ctypes.POINTER(_int), ctypes.POINTER(_f32p)],
+    "xad_image_free": [_f32p],
+    "xad_image_save": [ctypes.c_char_p, _int, _int, _vp],
+    "xad_image_test_pattern": [_int, _int, _vp],
+    "xad_trainer_create": [_vp, _int, _int, _vp, ctypes.POINTER(_vp)],
+    "xad_trainer_destroy": [_vp],
+    "xad_trainer_run": [_vp, _int, ctypes.POINTER(ctypes.c_double)],
+    "xad_trainer_iteration": [_vp],
+    "xad_trainer_download_image": [_vp, _vp],
+    "xad_trainer_get_state": [_vp, _vp, _vp, _vp, _vp],
+    "xad_trainer_set_params": [_vp, _vp, _vp],
+    "xad_trainer_save_checkpoint": [_vp, ctypes.c_char_p],
+    "xad_trainer_load_checkpoint": [_vp, ctypes.c_char_p],
     "xad_linreg_gradient_f64": [_int, _sz, _sz, _vp, _vp, _vp, _vp, _vp, _vp, _vp],
     "xad_linreg_sgd_f64": [_sz, _vp, _vp, _vp, _vp, _int, _int, ctypes.c_double, ctypes.c_double, _u64, _vp, _vp],
     "xad_host_linreg_gradient_f64": [_sz, _sz, _vp, _vp, _vp, _vp, _vp, _vp],
@@ -56,7 +73,8 @@ SIGNATURES = {
     "xad_host_rng_bits": [_vp, _sz, _u64, _u64, _u64],
     "xad_host_rng_uniform_f32": [_vp, _sz, _u64, _u64, _flt, _flt],
 }
-_RESTYPE = {"xad_last_error": ctypes.c_char_p, "xad_source_digest": ctypes.c_char_p, "xad_splat_destroy": None}
+_RESTYPE = {"xad_last_error": ctypes.c_char_p, "xad_source_digest": ctypes.c_char_p, "xad_training_usage": ctypes.c_char_p,
+            "xad_training_config_defaults": None, "xad_image_free": None, "xad_trainer_destroy": None, "xad_splat_destroy": None}
 
 
 def load():

@@ -15,7 +15,9 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(HERE)
 CSRC = os.path.join(HERE, "csrc")
+TRAINER = os.path.join(CSRC, "trainer")
 LIB = os.path.join(HERE, "libxad_hip.so")
+TRAIN_BIN = os.path.join(HERE, "xad_splat_train")
 OBJ_DIR = os.path.join(HERE, "build")
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
@@ -41,7 +43,10 @@ FLAGS = [
 
 
 def sources():
-    return sorted(os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".hip"))
+    """Translation units of the library: the kernels and, under trainer/, the host-only front-end."""
+    units = [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".hip")]
+    units += [os.path.join(TRAINER, f) for f in os.listdir(TRAINER) if f.endswith((".hip", ".cpp")) and f != "train_main.cpp"]
+    return sorted(units)
 
 
 def source_digest():
@@ -52,7 +57,7 @@ def source_digest():
     files = []
     for base in (CSRC, os.path.join(ROOT, "include")):
         for dirpath, _, names in os.walk(base):
-            files += [os.path.join(dirpath, f) for f in names if f.endswith((".hip", ".cuh", ".h"))]
+            files += [os.path.join(dirpath, f) for f in names if f.endswith((".hip", ".cuh", ".h", ".cpp"))]
     for path in sorted(files):
         h.update(os.path.relpath(path, ROOT).encode())
         h.update(b"\0")
@@ -63,7 +68,7 @@ def source_digest():
 
 
 def _compile(src, digest):
-    obj = os.path.join(OBJ_DIR, os.path.basename(src) + ".o")
+    obj = os.path.join(OBJ_DIR, os.path.relpath(src, CSRC).replace(os.sep, "_") + ".o")
     cmd = [HIPCC, *FLAGS, "-DXAD_SOURCE_DIGEST=\"%s\"" % digest, "-c", src, "-o", obj]
     proc = subprocess.run(cmd, capture_output=True, text=True)
     noise = "is not a recognized feature for this target"
@@ -83,10 +88,16 @@ def build(verbose=False):
         for _, err in results:
             if err.strip():
                 print(err, file=sys.stderr)
-    link = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-fno-gpu-sanitize", "-o", LIB, *objs, "-lpthread"]
+    link = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-fno-gpu-sanitize", "-o", LIB, *objs, "-lpthread", "-lz"]
     proc = subprocess.run(link, capture_output=True, text=True)
     if proc.returncode != 0:
         raise RuntimeError("link failed:\n" + proc.stderr)
+    # the trainer program: plain C++ on the C ABI, finds the library next to itself
+    program = ["g++", "-std=c++17", "-O2", "-Wall", "-Wextra", os.path.join(TRAINER, "train_main.cpp"), "-o", TRAIN_BIN,
+               "-L" + HERE, "-lxad_hip", "-Wl,-rpath,$ORIGIN", "-Wl,-rpath-link," + os.path.join(os.path.dirname(os.path.dirname(HIPCC)), "lib")]
+    proc = subprocess.run(program, capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError("building xad_splat_train failed:\n" + proc.stderr)
     return LIB
 
 

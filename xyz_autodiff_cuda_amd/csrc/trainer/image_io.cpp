@@ -1,0 +1,306 @@
+#include "image_io.h"
+
+#include <zlib.h>
+
+#include <algorithm>
+#include <cctype>
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <memory>
+
+namespace xad_train {
+namespace {
+
+using Bytes = std::vector<unsigned char>;
+
+constexpr unsigned char kPngSignature[8] = {0x89, 'P', 'N', 'G', '\r', '\n', 0x1A, '\n'};
+constexpr std::size_t kMaxPixels = std::size_t(1) << 28;  // 16384 x 16384
+
+std::string read_file(const std::string& path, Bytes& out) {
+    std::unique_ptr<std::FILE, int (*)(std::FILE*)> f(std::fopen(path.c_str(), "rb"), &std::fclose);
+    if (!f) return "cannot open " + path;
+    unsigned char chunk[1 << 16];
+    std::size_t got;
+    while ((got = std::fread(chunk, 1, sizeof chunk, f.get())) > 0) out.insert(out.end(), chunk, chunk + got);
+    if (std::ferror(f.get())) return "read error on " + path;
+    return "";
+}
+
+std::string write_file(const std::string& path, const Bytes& data) {
+    std::unique_ptr<std::FILE, int (*)(std::FILE*)> f(std::fopen(path.c_str(), "wb"), &std::fclose);
+    if (!f) return "cannot create " + path;
+    if (std::fwrite(data.data(), 1, data.size(), f.get()) != data.size()) return "write error on " + path;
+    if (std::fflush(f.get()) != 0) return "write error on " + path;
+    return "";
+}
+
+std::uint32_t be32(const unsigned char* p) {
+    return (std::uint32_t(p[0]) << 24) | (std::uint32_t(p[1]) << 16) | (std::uint32_t(p[2]) << 8) | p[3];
+}
+
+void put_be32(Bytes& out, std::uint32_t v) {
+    for (int shift = 24; shift >= 0; shift -= 8) out.push_back(static_cast<unsigned char>(v >> shift));
+}
+
+// ---- PNG ---------------------------------------------------------------------
+
+int paeth(int a, int b, int c) {
+    const int p = a + b - c;
+    const int pa = std::abs(p - a), pb = std::abs(p - b), pc = std::abs(p - c);
+    if (pa <= pb && pa <= pc) return a;
+    return pb <= pc ? b : c;
+}
+
+// Undoes the per-row prediction filters in place; `raw` holds height rows of
+// 1 + row_bytes bytes.  Returns false on an unknown filter type.
+bool unfilter(Bytes& raw, std::size_t height, std::size_t row_bytes, std::size_t bpp) {
+    const Bytes zero_row(row_bytes, 0);
+    for (std::size_t y = 0; y < height; ++y) {
+        unsigned char* row = raw.data() + y * (row_bytes + 1) + 1;
+        const unsigned char* up = y ? row - (row_bytes + 1) : zero_row.data();
+        const int type = row[-1];
+        for (std::size_t i = 0; i < row_bytes; ++i) {
+            const int a = i >= bpp ? row[i - bpp] : 0;
+            const int b = up[i];
+            const int c = i >= bpp ? up[i - bpp] : 0;
+            int predicted;
+            switch (type) {
+                case 0: predicted = 0; break;
+                case 1: predicted = a; break;
+                case 2: predicted = b; break;
+                case 3: predicted = (a + b) >> 1; break;
+                case 4: predicted = paeth(a, b, c); break;
+                default: return false;
+            }
+            row[i] = static_cast<unsigned char>(row[i] + predicted);
+        }
+    }
+    return true;
+}
+
+std::string decode_png(const Bytes& file, Image& out) {
+    std::size_t pos = 8;
+    std::uint32_t width = 0, height = 0;
+    int depth = 0, colour = -1;
+    Bytes palette, compressed;
+    bool seen_end = false;
+    while (!seen_end) {
+        if (pos + 12 > file.size()) return "PNG: truncated file";
+        const std::uint32_t length = be32(&file[pos]);
+        if (length > file.size() - pos - 12) return "PNG: chunk runs past the end of the file";
+        const unsigned char* type = &file[pos + 4];
+        const unsigned char* data = &file[pos + 8];
+        if (be32(data + length) != crc32(0, type, length + 4)) return "PNG: chunk checksum mismatch";
+        if (!std::memcmp(type, "IHDR", 4)) {
+            if (length != 13) return "PNG: bad header chunk";
+            width = be32(data);
+            height = be32(data + 4);
+            depth = data[8];
+            colour = data[9];
+            if (data[10] != 0 || data[11] != 0) return "PNG: unknown compression or filter method";
+            if (data[12] != 0) return "PNG: interlaced files are not supported";
+        } else if (colour < 0) {
+            return "PNG: first chunk is not the header";
+        } else if (!std::memcmp(type, "PLTE", 4)) {
+            palette.assign(data, data + length);
+        } else if (!std::memcmp(type, "IDAT", 4)) {
+            compressed.insert(compressed.end(), data, data + length);
+        } else if (!std::memcmp(type, "IEND", 4)) {
+            seen_end = true;
+        } else if (!(type[0] & 0x20)) {
+            return "PNG: unknown critical chunk";
+        }
+        pos += 12 + length;
+    }
+    int channels;
+    switch (colour) {
+        case 0: channels = 1; break;
+        case 2: channels = 3; break;
+        case 3: channels = 1; break;
+        case 4: channels = 2; break;
+        case 6: channels = 4; break;
+        default: return "PNG: unknown colour type";
+    }
+    const bool depth_ok = colour == 0   ? (depth == 1 || depth == 2 || depth == 4 || depth == 8 || depth == 16)
+                          : colour == 3 ? (depth == 1 || depth == 2 || depth == 4 || depth == 8)
+                                        : (depth == 8 || depth == 16);
+    if (!depth_ok) return "PNG: bit depth not allowed for this colour type";
+    if (width == 0 || height == 0 || std::size_t(width) * height > kMaxPixels) return "PNG: unreasonable image size";
+    if (colour == 3 && (palette.empty() || palette.size() % 3)) return "PNG: palette missing or malformed";
+
+    const std::size_t row_bytes = (std::size_t(width) * channels * depth + 7) / 8;
+    Bytes raw(std::size_t(height) * (row_bytes + 1));
+    uLongf raw_size = raw.size();
+    const int z = uncompress(raw.data(), &raw_size, compressed.data(), compressed.size());
+    if (z != Z_OK || raw_size != raw.size()) return "PNG: image data does not inflate to the declared size";
+    if (!unfilter(raw, height, row_bytes, std::max<std::size_t>(1, std::size_t(channels) * depth / 8)))
+        return "PNG: unknown row filter";
+
+    out.width = static_cast<int>(width);
+    out.height = static_cast<int>(height);
+    out.rgb.assign(std::size_t(width) * height * 3, 0.0f);
+    const float max_sample = static_cast<float>((1u << depth) - 1);
+    for (std::size_t y = 0; y < height; ++y) {
+        const unsigned char* row = raw.data() + y * (row_bytes + 1) + 1;
+        auto sample = [&](std::size_t index) -> unsigned {
+            if (depth == 8) return row[index];
+            if (depth == 16) return (unsigned(row[2 * index]) << 8) | row[2 * index + 1];
+            const std::size_t bit = index * depth;
+            return (row[bit >> 3] >> (8 - depth - (bit & 7))) & ((1u << depth) - 1);
+        };
+        for (std::size_t x = 0; x < width; ++x) {
+            float* px = &out.rgb[(y * width + x) * 3];
+            if (colour == 3) {
+                const unsigned entry = sample(x);
+                if (3 * entry + 2 >= palette.size()) return "PNG: palette index out of range";
+                for (int c = 0; c < 3; ++c) px[c] = palette[3 * entry + c] / 255.0f;
+            } else if (channels <= 2) {
+                px[0] = px[1] = px[2] = sample(x * channels) / max_sample;
+            } else {
+                for (int c = 0; c < 3; ++c) px[c] = sample(x * channels + c) / max_sample;
+            }
+        }
+    }
+    return "";
+}
+
+void append_chunk(Bytes& out, const char* type, const Bytes& data) {
+    put_be32(out, static_cast<std::uint32_t>(data.size()));
+    const std::size_t start = out.size();
+    out.insert(out.end(), type, type + 4);
+    out.insert(out.end(), data.begin(), data.end());
+    put_be32(out, static_cast<std::uint32_t>(crc32(0, out.data() + start, static_cast<uInt>(out.size() - start))));
+}
+
+std::string encode_png(int width, int height, const Bytes& pixels, Bytes& out) {
+    const std::size_t row_bytes = std::size_t(width) * 3;
+    Bytes raw;
+    raw.reserve(std::size_t(height) * (row_bytes + 1));
+    for (int y = 0; y < height; ++y) {
+        raw.push_back(0);  // filter: none
+        raw.insert(raw.end(), pixels.begin() + y * row_bytes, pixels.begin() + (y + 1) * row_bytes);
+    }
+    uLongf packed_size = compressBound(raw.size());
+    Bytes packed(packed_size);
+    if (compress2(packed.data(), &packed_size, raw.data(), raw.size(), 6) != Z_OK) return "PNG: deflate failed";
+    packed.resize(packed_size);
+
+    out.assign(kPngSignature, kPngSignature + 8);
+    Bytes header;
+    put_be32(header, static_cast<std::uint32_t>(width));
+    put_be32(header, static_cast<std::uint32_t>(height));
+    const unsigned char tail[5] = {8, 2, 0, 0, 0};  // 8 bits, RGB, deflate, adaptive filters, not interlaced
+    header.insert(header.end(), tail, tail + 5);
+    append_chunk(out, "IHDR", header);
+    append_chunk(out, "IDAT", packed);
+    append_chunk(out, "IEND", Bytes());
+    return "";
+}
+
+// ---- PPM / PGM -----------------------------------------------------------------
+
+// Next unsigned integer of a netpbm header, skipping white space and # comments.
+bool next_header_number(const Bytes& file, std::size_t& pos, unsigned& value) {
+    for (;;) {
+        while (pos < file.size() && std::isspace(file[pos])) ++pos;
+        if (pos < file.size() && file[pos] == '#') {
+            while (pos < file.size() && file[pos] != '\n') ++pos;
+            continue;
+        }
+        break;
+    }
+    if (pos >= file.size() || !std::isdigit(file[pos])) return false;
+    unsigned long v = 0;
+    while (pos < file.size() && std::isdigit(file[pos])) {
+        v = v * 10 + (file[pos++] - '0');
+        if (v > 1000000000ul) return false;
+    }
+    value = static_cast<unsigned>(v);
+    return true;
+}
+
+std::string decode_netpbm(const Bytes& file, Image& out) {
+    const int channels = file[1] == '6' ? 3 : 1;
+    std::size_t pos = 2;
+    unsigned width, height, max_value;
+    if (!next_header_number(file, pos, width) || !next_header_number(file, pos, height) ||
+        !next_header_number(file, pos, max_value))
+        return "PPM: malformed header";
+    if (pos >= file.size() || !std::isspace(file[pos])) return "PPM: malformed header";
+    ++pos;  // the single white-space byte before the raster
+    if (max_value == 0 || max_value > 65535) return "PPM: maximum value out of range";
+    if (width == 0 || height == 0 || std::size_t(width) * height > kMaxPixels) return "PPM: unreasonable image size";
+    const std::size_t sample_bytes = max_value > 255 ? 2 : 1;
+    const std::size_t samples = std::size_t(width) * height * channels;
+    if (file.size() - pos < samples * sample_bytes) return "PPM: raster is shorter than the header declares";
+    out.width = static_cast<int>(width);
+    out.height = static_cast<int>(height);
+    out.rgb.resize(std::size_t(width) * height * 3);
+    const unsigned char* raster = file.data() + pos;
+    for (std::size_t i = 0; i < std::size_t(width) * height; ++i) {
+        for (int c = 0; c < 3; ++c) {
+            const std::size_t s = i * channels + (channels == 3 ? c : 0);
+            const unsigned v = sample_bytes == 2 ? (unsigned(raster[2 * s]) << 8) | raster[2 * s + 1] : raster[s];
+            out.rgb[i * 3 + c] = static_cast<float>(v) / static_cast<float>(max_value);
+        }
+    }
+    return "";
+}
+
+bool ends_with(const std::string& s, const char* suffix) {
+    const std::size_t n = std::strlen(suffix);
+    if (s.size() < n) return false;
+    for (std::size_t i = 0; i < n; ++i)
+        if (std::tolower(static_cast<unsigned char>(s[s.size() - n + i])) != suffix[i]) return false;
+    return true;
+}
+
+}  // namespace
+
+std::string load_image(const std::string& path, Image& out) {
+    Bytes file;
+    if (std::string err = read_file(path, file); !err.empty()) return err;
+    if (file.size() >= 8 && !std::memcmp(file.data(), kPngSignature, 8)) return decode_png(file, out);
+    if (file.size() >= 3 && file[0] == 'P' && (file[1] == '6' || file[1] == '5')) return decode_netpbm(file, out);
+    if (file.size() >= 2 && file[0] == 0xFF && file[1] == 0xD8) return "JPEG files are not supported; convert " + path + " to PNG or PPM";
+    return path + " is neither a PNG nor a binary PPM/PGM file";
+}
+
+std::string save_image(const std::string& path, int width, int height, const float* rgb) {
+    if (width <= 0 || height <= 0 || !rgb) return "save_image: empty image";
+    Bytes pixels(std::size_t(width) * height * 3);
+    for (std::size_t i = 0; i < pixels.size(); ++i) {
+        const float v = rgb[i];
+        const float clamped = v > 0.0f ? (v < 1.0f ? v : 1.0f) : 0.0f;  // NaN becomes 0
+        pixels[i] = static_cast<unsigned char>(clamped * 255.0f + 0.5f);
+    }
+    Bytes file;
+    if (ends_with(path, ".png")) {
+        if (std::string err = encode_png(width, height, pixels, file); !err.empty()) return err;
+    } else if (ends_with(path, ".ppm")) {
+        char header[64];
+        const int n = std::snprintf(header, sizeof header, "P6\n%d %d\n255\n", width, height);
+        file.assign(header, header + n);
+        file.insert(file.end(), pixels.begin(), pixels.end());
+    } else {
+        return "save_image: " + path + " must end in .png or .ppm";
+    }
+    return write_file(path, file);
+}
+
+void test_pattern(int width, int height, float* rgb) {
+    for (int y = 0; y < height; ++y) {
+        for (int x = 0; x < width; ++x) {
+            const float r = static_cast<float>(x) / width;
+            const float g = static_cast<float>(y) / height;
+            float* px = rgb + (std::size_t(y) * width + x) * 3;
+            px[0] = r;
+            px[1] = g;
+            px[2] = 0.5f * (r + g);
+        }
+    }
+}
+
+}  // namespace xad_train

@@ -1,0 +1,273 @@
+// Training run of the splatting example on the current device, and the C ABI
+// of the trainer front-end (images, checkpoints).
+//
+// Host-side counterpart of GaussianSplattingTrainer and GaussianCollection of
+// xyz-autodiff-cuda (examples/mini-gaussian-splatting/gaussian_splatting_training.cu:14-181,
+// gaussian_parameters.cu:9-116): it owns the device state and drives
+// xad_splat_step and xad_adam_step_f32; all arithmetic happens there.
+#include <cmath>
+#include <cstdlib>
+#include <cstring>
+#include <new>
+#include <string>
+#include <vector>
+
+#include "../common.cuh"
+#include "../rng.cuh"
+#include "checkpoint.h"
+#include "image_io.h"
+
+struct xad_trainer {
+    xad_training_config config;
+    int width = 0, height = 0, gaussians = 0;
+    int iteration = 0;
+    int device = 0;
+    hipStream_t stream = nullptr;
+    xad_splat_context* splat = nullptr;
+    // one allocation: params | grads | m | v (9G each) | depth (G)
+    float* state = nullptr;
+    float* target = nullptr;
+    float* image = nullptr;
+
+    std::size_t g() const { return static_cast<std::size_t>(gaussians); }
+    std::size_t pixels() const { return static_cast<std::size_t>(width) * height; }
+    float* params() const { return state; }
+    float* grads() const { return state + 9 * g(); }
+    float* m() const { return state + 18 * g(); }
+    float* v() const { return state + 27 * g(); }
+    float* depth() const { return state + 36 * g(); }
+};
+
+namespace {
+
+// Initial values of GaussianCollection::initialize_random
+// (gaussian_parameters.cu:27-66), one random stream per row.
+void initial_gaussians(const xad_trainer& t, std::vector<float>& params, std::vector<float>& depth) {
+    const std::size_t g = t.g();
+    params.assign(9 * g, 0.0f);
+    depth.assign(g, 0.0f);
+    struct Row { int row; float lo, hi; };
+    const Row rows[] = {{0, 0.0f, static_cast<float>(t.width)}, {1, 0.0f, static_cast<float>(t.height)},
+                        {2, 0.0f, 2.0f}, {3, 0.0f, 2.0f},
+                        {5, 0.1f, 0.2f}, {6, 0.1f, 0.2f}, {7, 0.1f, 0.2f}, {8, 0.05f, 0.1f}};
+    for (const Row& r : rows) {
+        const std::uint64_t key = xad_rng::stream_key(t.config.seed, static_cast<std::uint64_t>(r.row));
+        for (std::size_t i = 0; i < g; ++i) {
+            float value = xad_rng::uniform(xad_rng::bits(key, i), r.lo, r.hi);
+            if (r.row == 2 || r.row == 3) value = std::fmax(1.0f, value);
+            params[r.row * g + i] = value;
+        }
+    }
+    const std::uint64_t key = xad_rng::stream_key(t.config.seed, 9);
+    for (std::size_t i = 0; i < g; ++i) depth[i] = xad_rng::unit_float(xad_rng::bits(key, i));
+}
+
+int bind_device(const xad_trainer* t) {
+    XAD_HIP_TRY(hipSetDevice(t->device));
+    return XAD_OK;
+}
+
+int upload(const xad_trainer* t, float* dst, const float* src, std::size_t count) {
+    XAD_HIP_TRY(hipMemcpyAsync(dst, src, count * sizeof(float), hipMemcpyHostToDevice, t->stream));
+    XAD_HIP_TRY(hipStreamSynchronize(t->stream));
+    return XAD_OK;
+}
+
+int download(const xad_trainer* t, float* dst, const float* src, std::size_t count) {
+    XAD_HIP_TRY(hipMemcpyAsync(dst, src, count * sizeof(float), hipMemcpyDeviceToHost, t->stream));
+    XAD_HIP_TRY(hipStreamSynchronize(t->stream));
+    return XAD_OK;
+}
+
+int create(const xad_training_config* config, int width, int height, const float* target_rgb, xad_trainer* t) {
+    t->config = *config;
+    t->width = width;
+    t->height = height;
+    t->gaussians = config->num_gaussians;
+    XAD_HIP_TRY(hipGetDevice(&t->device));
+    XAD_HIP_TRY(hipStreamCreate(&t->stream));
+    if (int st = xad_splat_create(width, height, t->gaussians, 0, &t->splat)) return st;
+    XAD_HIP_TRY(hipMalloc(&t->state, 37 * t->g() * sizeof(float)));
+    XAD_HIP_TRY(hipMalloc(&t->target, 3 * t->pixels() * sizeof(float)));
+    XAD_HIP_TRY(hipMalloc(&t->image, 3 * t->pixels() * sizeof(float)));
+    XAD_HIP_TRY(hipMemsetAsync(t->state, 0, 37 * t->g() * sizeof(float), t->stream));
+    XAD_HIP_TRY(hipMemsetAsync(t->image, 0, 3 * t->pixels() * sizeof(float), t->stream));
+    std::vector<float> params, depth;
+    initial_gaussians(*t, params, depth);
+    if (int st = upload(t, t->params(), params.data(), params.size())) return st;
+    if (int st = upload(t, t->depth(), depth.data(), depth.size())) return st;
+    return upload(t, t->target, target_rgb, 3 * t->pixels());
+}
+
+}  // namespace
+
+extern "C" int xad_trainer_create(const xad_training_config* config, int width, int height, const float* target_rgb,
+                                  xad_trainer** out) {
+    XAD_REQUIRE(config && target_rgb && out, "config, target_rgb and out must not be null");
+    XAD_REQUIRE(width > 0 && height > 0, "image size must be positive, got %d x %d", width, height);
+    XAD_REQUIRE(config->num_gaussians > 0, "Number of Gaussians must be positive");
+    XAD_REQUIRE(config->lr_center > 0 && config->lr_scale > 0 && config->lr_rotation > 0 && config->lr_color > 0 &&
+                    config->lr_opacity > 0,
+                "All learning rates must be positive");
+    XAD_REQUIRE(config->beta1 > 0 && config->beta1 < 1, "Beta1 must be in range (0, 1)");
+    XAD_REQUIRE(config->beta2 > 0 && config->beta2 < 1, "Beta2 must be in range (0, 1)");
+    XAD_REQUIRE(config->epsilon > 0, "Epsilon must be positive");
+    *out = nullptr;
+    xad_trainer* t = new (std::nothrow) xad_trainer();
+    XAD_REQUIRE(t, "out of host memory");
+    const int status = create(config, width, height, target_rgb, t);
+    if (status != XAD_OK) {
+        // keep the message of the failure, not of the clean-up
+        const std::string message = xad_last_error();
+        xad_trainer_destroy(t);
+        return xad::fail(status, "%s", message.c_str());
+    }
+    *out = t;
+    return XAD_OK;
+}
+
+extern "C" void xad_trainer_destroy(xad_trainer* t) {
+    if (!t) return;
+    (void)hipSetDevice(t->device);
+    if (t->stream) (void)hipStreamSynchronize(t->stream);
+    if (t->splat) xad_splat_destroy(t->splat);
+    if (t->state) (void)hipFree(t->state);
+    if (t->target) (void)hipFree(t->target);
+    if (t->image) (void)hipFree(t->image);
+    if (t->stream) (void)hipStreamDestroy(t->stream);
+    delete t;
+}
+
+extern "C" int xad_trainer_run(xad_trainer* t, int iterations, double* loss_out) {
+    XAD_REQUIRE(t, "trainer must not be null");
+    XAD_REQUIRE(iterations >= 0, "iterations must not be negative");
+    if (int st = bind_device(t)) return st;
+    const xad_training_config& c = t->config;
+    const float learning_rates[9] = {c.lr_center, c.lr_center, c.lr_scale, c.lr_scale, c.lr_rotation,
+                                     c.lr_color,  c.lr_color,  c.lr_color, c.lr_opacity};
+    for (int i = 0; i < iterations; ++i) {
+        double* loss = (i + 1 == iterations) ? loss_out : nullptr;
+        if (int st = xad_splat_step(t->splat, t->params(), t->depth(), t->target, t->image, t->grads(), loss, t->stream))
+            return st;
+        if (int st = xad_adam_step_f32(t->g(), 9, t->params(), t->grads(), t->m(), t->v(), learning_rates, c.beta1,
+                                       c.beta2, c.epsilon, t->iteration + 1, t->stream))
+            return st;
+        ++t->iteration;
+    }
+    XAD_HIP_TRY(hipStreamSynchronize(t->stream));
+    return XAD_OK;
+}
+
+extern "C" int xad_trainer_iteration(const xad_trainer* t) { return t ? t->iteration : -1; }
+
+extern "C" int xad_trainer_download_image(xad_trainer* t, float* rgb) {
+    XAD_REQUIRE(t && rgb, "trainer and rgb must not be null");
+    if (int st = bind_device(t)) return st;
+    return download(t, rgb, t->image, 3 * t->pixels());
+}
+
+extern "C" int xad_trainer_get_state(xad_trainer* t, float* params, float* m, float* v, float* depth) {
+    XAD_REQUIRE(t, "trainer must not be null");
+    if (int st = bind_device(t)) return st;
+    if (params)
+        if (int st = download(t, params, t->params(), 9 * t->g())) return st;
+    if (m)
+        if (int st = download(t, m, t->m(), 9 * t->g())) return st;
+    if (v)
+        if (int st = download(t, v, t->v(), 9 * t->g())) return st;
+    if (depth)
+        if (int st = download(t, depth, t->depth(), t->g())) return st;
+    return XAD_OK;
+}
+
+extern "C" int xad_trainer_set_params(xad_trainer* t, const float* params, const float* depth) {
+    XAD_REQUIRE(t, "trainer must not be null");
+    if (int st = bind_device(t)) return st;
+    if (params)
+        if (int st = upload(t, t->params(), params, 9 * t->g())) return st;
+    if (depth)
+        if (int st = upload(t, t->depth(), depth, t->g())) return st;
+    return XAD_OK;
+}
+
+extern "C" int xad_trainer_save_checkpoint(xad_trainer* t, const char* path) {
+    XAD_REQUIRE(t && path && path[0], "trainer and path must not be null or empty");
+    if (int st = bind_device(t)) return st;
+    xad_train::CheckpointState state;
+    xad_train::CheckpointHeader& h = state.header;
+    std::memset(&h, 0, sizeof h);
+    h.width = t->width;
+    h.height = t->height;
+    h.num_gaussians = t->gaussians;
+    h.iteration = t->iteration;
+    h.lr_center = t->config.lr_center;
+    h.lr_scale = t->config.lr_scale;
+    h.lr_rotation = t->config.lr_rotation;
+    h.lr_color = t->config.lr_color;
+    h.lr_opacity = t->config.lr_opacity;
+    h.beta1 = t->config.beta1;
+    h.beta2 = t->config.beta2;
+    h.epsilon = t->config.epsilon;
+    h.seed = t->config.seed;
+    state.params.resize(9 * t->g());
+    state.m.resize(9 * t->g());
+    state.v.resize(9 * t->g());
+    state.depth.resize(t->g());
+    if (int st = xad_trainer_get_state(t, state.params.data(), state.m.data(), state.v.data(), state.depth.data()))
+        return st;
+    const std::string err = xad_train::write_checkpoint(path, state);
+    XAD_REQUIRE(err.empty(), "%s", err.c_str());
+    return XAD_OK;
+}
+
+extern "C" int xad_trainer_load_checkpoint(xad_trainer* t, const char* path) {
+    XAD_REQUIRE(t && path && path[0], "trainer and path must not be null or empty");
+    if (int st = bind_device(t)) return st;
+    xad_train::CheckpointState state;
+    const std::string err = xad_train::read_checkpoint(path, state);
+    XAD_REQUIRE(err.empty(), "%s", err.c_str());
+    const xad_train::CheckpointHeader& h = state.header;
+    XAD_REQUIRE(h.num_gaussians == t->gaussians, "checkpoint holds %d Gaussians, the trainer %d", h.num_gaussians,
+                t->gaussians);
+    XAD_REQUIRE(h.width == t->width && h.height == t->height, "checkpoint is for a %d x %d image, the trainer for %d x %d",
+                h.width, h.height, t->width, t->height);
+    if (int st = upload(t, t->params(), state.params.data(), state.params.size())) return st;
+    if (int st = upload(t, t->m(), state.m.data(), state.m.size())) return st;
+    if (int st = upload(t, t->v(), state.v.data(), state.v.size())) return st;
+    if (int st = upload(t, t->depth(), state.depth.data(), state.depth.size())) return st;
+    t->iteration = h.iteration;
+    return XAD_OK;
+}
+
+// ---- images ----------------------------------------------------------------------
+
+extern "C" int xad_image_load(const char* path, int* width, int* height, float** rgb) {
+    XAD_REQUIRE(path && width && height && rgb, "path, width, height and rgb must not be null");
+    xad_train::Image image;
+    const std::string err = xad_train::load_image(path, image);
+    XAD_REQUIRE(err.empty(), "%s", err.c_str());
+    float* copy = static_cast<float*>(std::malloc(image.rgb.size() * sizeof(float)));
+    XAD_REQUIRE(copy, "out of host memory");
+    std::memcpy(copy, image.rgb.data(), image.rgb.size() * sizeof(float));
+    *width = image.width;
+    *height = image.height;
+    *rgb = copy;
+    return XAD_OK;
+}
+
+extern "C" void xad_image_free(float* rgb) { std::free(rgb); }
+
+extern "C" int xad_image_save(const char* path, int width, int height, const float* rgb) {
+    XAD_REQUIRE(path && rgb, "path and rgb must not be null");
+    XAD_REQUIRE(width > 0 && height > 0, "image size must be positive, got %d x %d", width, height);
+    const std::string err = xad_train::save_image(path, width, height, rgb);
+    XAD_REQUIRE(err.empty(), "%s", err.c_str());
+    return XAD_OK;
+}
+
+extern "C" int xad_image_test_pattern(int width, int height, float* rgb) {
+    XAD_REQUIRE(rgb, "rgb must not be null");
+    XAD_REQUIRE(width > 0 && height > 0, "image size must be positive, got %d x %d", width, height);
+    xad_train::test_pattern(width, height, rgb);
+    return XAD_OK;
+}
