@@ -44,5 +44,7 @@ struct TileRect {
 // Gradient of the loss with respect to the fields of a Record the parameters
 // reach: centre (2), inverse covariance (3), colour (3), alpha0 (1).
 constexpr int kRecordGrads = 9;
+// Rows of the accumulator are 64 bytes apart, so the atomics on one Gaussian stay in one cache line.
+constexpr int kRecordGradStride = 16;
 
 }  // namespace xad_splat

@@ -137,7 +137,7 @@ extern "C" int xad_splat_create(int width, int height, int num_gaussians, std::s
     alloc(&c->range_begin, sizeof(std::uint32_t) * c->tiles * 2);
     alloc(&c->final_T, sizeof(float) * pixels);
     alloc(&c->n_contrib, sizeof(std::uint32_t) * pixels);
-    alloc(&c->record_grads, sizeof(float) * G * kRecordGrads);
+    alloc(&c->record_grads, sizeof(float) * G * kRecordGradStride);
     alloc(&c->loss, sizeof(double));
     if (st == XAD_OK) {
         c->range_end = c->range_begin + c->tiles;
@@ -214,7 +214,7 @@ extern "C" int xad_splat_step(xad_splat_context* c, const float* params, const f
                                        image, c->final_T, c->n_contrib))
         return st;
     mark(c, 5, s);
-    XAD_HIP_TRY(hipMemsetAsync(c->record_grads, 0, sizeof(float) * static_cast<std::size_t>(c->G) * kRecordGrads, s));
+    XAD_HIP_TRY(hipMemsetAsync(c->record_grads, 0, sizeof(float) * static_cast<std::size_t>(c->G) * kRecordGradStride, s));
     XAD_HIP_TRY(hipMemsetAsync(c->loss, 0, sizeof(double), s));
     if (int st = launch_render_backward(s, c->width, c->height, c->range_begin, c->range_end, c->ids_sorted, c->records,
                                         image, target, c->final_T, c->n_contrib, c->record_grads, c->loss))

@@ -178,12 +178,6 @@ __device__ __forceinline__ Staged stage_record(const Record* __restrict__ record
     return s;
 }
 
-__device__ __forceinline__ float falloff_of(const Staged& r, float dx, float dy) {
-    const float t = ::fmaf(r.b2_s, dy, r.a_s * dx);
-    const float q_scaled = ::fmaf(r.c_s * dy, dy, t * dx);
-    return math::fp32::exp2_raw(q_scaled);
-}
-
 __device__ __forceinline__ std::uint32_t wave_max(std::uint32_t v) {
     // 64-lane maximum through the LDS crossbar-free DPP path: rows, then row heads
     auto step = [](std::uint32_t x, auto ctrl) {
@@ -215,6 +209,7 @@ __global__ void __launch_bounds__(kChunk) render_forward_kernel(
     const int x0 = (tile % tiles_x) * kTile + (lane & 3) * kLanePixels;
     const int y = (tile / tiles_x) * kTile + (lane >> 2);
     const float py = static_cast<float>(y);
+    const float px0 = static_cast<float>(x0);
 
     const std::uint32_t first = range_begin[tile], last = range_end[tile];
     float T[kLanePixels], red[kLanePixels], green[kLanePixels], blue[kLanePixels];
@@ -235,13 +230,17 @@ __global__ void __launch_bounds__(kChunk) render_forward_kernel(
         const int count = static_cast<int>(last - base < kChunk ? last - base : kChunk);
         for (int j = 0; j < count; ++j) {
             const Staged r = staged[j];
+            // exponent of the falloff as a polynomial in dx: (a_s dx + e) dx + f
             const float dy = py - r.cy;
+            const float e = r.b2_s * dy;
+            const float f = r.c_s * dy * dy;
+            const float dx0 = px0 - r.cx;
 #pragma unroll
             for (int p = 0; p < kLanePixels; ++p) {
                 // a pixel stops, for good, before the first Gaussian it meets with T below the threshold
                 done[p] = done[p] || T[p] < kMinTransmittance;
-                const float dx = static_cast<float>(x0 + p) - r.cx;
-                const float a = falloff_of(r, dx, dy) * r.alpha0;
+                const float dx = dx0 + static_cast<float>(p);
+                const float a = math::fp32::exp2_raw(::fmaf(::fmaf(r.a_s, dx, e), dx, f)) * r.alpha0;
                 const float alpha = done[p] ? 0.f : (a > kAlphaMax ? kAlphaMax : a);
                 const float weight = T[p] * alpha;
                 red[p] = ::fmaf(weight, r.red, red[p]);
@@ -335,17 +334,20 @@ __global__ void __launch_bounds__(kChunk) render_backward_kernel(
     const int y = (tile / tiles_x) * kTile + (lane >> 2);
     const float py = static_cast<float>(y);
 
-    float dC[kLanePixels][3], T[kLanePixels], behind[kLanePixels][3], last_alpha[kLanePixels];
+    // Per pixel: dC = d loss / d colour, T = transmittance behind the Gaussian the walk is at,
+    // D = -dC . (colour composited behind that Gaussian), in absolute (not normalised) terms.  (Kept
+    // negated so that no negated reciprocal is needed: the compiler would compute one separately.)
+    float dC[kLanePixels][3], T[kLanePixels], D[kLanePixels];
     std::uint32_t used[kLanePixels];
     float my_loss = 0.f;
     std::uint32_t my_max = 0;
 #pragma unroll
     for (int p = 0; p < kLanePixels; ++p) {
         T[p] = 1.f;
+        D[p] = 0.f;
         used[p] = 0;
-        last_alpha[p] = 0.f;
 #pragma unroll
-        for (int c = 0; c < 3; ++c) dC[p][c] = behind[p][c] = 0.f;
+        for (int c = 0; c < 3; ++c) dC[p][c] = 0.f;
         if (x0 + p < width && y < height) {
             const std::size_t at = static_cast<std::size_t>(y) * width + x0 + p;
 #pragma unroll
@@ -366,7 +368,7 @@ __global__ void __launch_bounds__(kChunk) render_backward_kernel(
     const std::uint32_t deepest = wave_max(my_max);  // entries [0, deepest) were composited by some pixel
     if (deepest == 0) return;
     const std::uint32_t first = range_begin[tile];
-    float last_col[3] = {0.f, 0.f, 0.f};
+    const float px0 = static_cast<float>(x0);
 
     for (std::uint32_t chunk = (deepest + kChunk - 1) / kChunk; chunk-- > 0;) {
         const std::uint32_t chunk_first = chunk * kChunk;
@@ -382,44 +384,46 @@ __global__ void __launch_bounds__(kChunk) render_backward_kernel(
         for (int j = count - 1; j >= 0; --j) {
             const std::uint32_t position = chunk_first + j;
             const Staged r = staged[j];
+            // exponent of the falloff as a polynomial in dx: (a_s dx + e) dx + f
             const float dy = py - r.cy;
-            const float g_q_scale = -0.5f * r.alpha0;
-            float v[9] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+            const float e = r.b2_s * dy;
+            const float f = r.c_s * dy * dy;
+            const float dx0 = px0 - r.cx;
+            float through[kLanePixels];  // d loss / d alpha0 of this Gaussian, per pixel
+            float colour[3] = {0.f, 0.f, 0.f};
 #pragma unroll
             for (int p = 0; p < kLanePixels; ++p) {
                 // A pixel is idle until the walk reaches the last Gaussian it composited, and
-                // active from there on.  While idle, alpha = 0 leaves T, `behind` and
-                // last_alpha at their initial values, so no branch is needed.
+                // active from there on.  While idle, alpha = 0 leaves T and D at their initial
+                // values, so no branch is needed.
                 const bool active = position < used[p];
-                const float dx = static_cast<float>(x0 + p) - r.cx;
-                const float falloff = falloff_of(r, dx, dy);
+                const float dx = dx0 + static_cast<float>(p);
+                const float falloff = math::fp32::exp2_raw(::fmaf(::fmaf(r.a_s, dx, e), dx, f));
                 const float a = falloff * r.alpha0;
                 const bool clamped = a > kAlphaMax;
                 const float alpha = active ? (clamped ? kAlphaMax : a) : 0.f;
-                T[p] = T[p] * __builtin_amdgcn_rcpf(1.f - alpha);  // transmittance in front of this Gaussian
-                float d_alpha = 0.f;
-                const float col[3] = {r.red, r.green, r.blue};
-                const float weight = alpha * T[p];
+                const float inv = __builtin_amdgcn_rcpf(1.f - alpha);
+                const float T_front = T[p] * inv;  // transmittance in front of this Gaussian
+                const float dot = ::fmaf(dC[p][2], r.blue, ::fmaf(dC[p][1], r.green, dC[p][0] * r.red));
+                // d loss / d alpha = T_front (dC . colour) - (dC . colour behind) / (1 - alpha)
+                //                  = T_front dot + D inv
+                const float d_alpha = ::fmaf(D[p], inv, T_front * dot);
+                const float weight = alpha * T_front;
+                D[p] = ::fmaf(-weight, dot, D[p]);
+                T[p] = T_front;
 #pragma unroll
-                for (int c = 0; c < 3; ++c) {
-                    behind[p][c] = ::fmaf(last_alpha[p], last_col[c] - behind[p][c], behind[p][c]);
-                    d_alpha = ::fmaf(col[c] - behind[p][c], dC[p][c], d_alpha);
-                    v[5 + c] = ::fmaf(weight, dC[p][c], v[5 + c]);
-                }
-                last_alpha[p] = alpha;
-                const float through = (active && !clamped) ? d_alpha * T[p] * falloff : 0.f;  // d loss / d alpha0
-                v[8] += through;
-                const float g_q = through * g_q_scale;
-                const float gx = g_q * dx, gy = g_q * dy;
-                v[0] += gx;
-                v[1] += gy;
-                v[2] = ::fmaf(gx, dx, v[2]);
-                v[3] = ::fmaf(gx, dy, v[3]);
-                v[4] = ::fmaf(gy, dy, v[4]);
+                for (int c = 0; c < 3; ++c) colour[c] = ::fmaf(weight, dC[p][c], colour[c]);
+                through[p] = (active && !clamped) ? d_alpha * falloff : 0.f;
             }
-            last_col[0] = r.red;
-            last_col[1] = r.green;
-            last_col[2] = r.blue;
+            // Moments of `through` over the lane's four pixels (offsets 0..3 from dx0) give the five
+            // sums  sum t dx^i dy^j  the Mahalanobis backward rule needs; their common factor
+            // d alpha / d q / falloff = -alpha0 / 2 is applied once per Gaussian below.
+            const float m0 = (through[0] + through[1]) + (through[2] + through[3]);
+            const float m1 = ::fmaf(3.f, through[3], ::fmaf(2.f, through[2], through[1]));
+            const float m2 = ::fmaf(9.f, through[3], ::fmaf(4.f, through[2], through[1]));
+            const float sx = ::fmaf(dx0, m0, m1);
+            const float sy = dy * m0;
+            const float v[9] = {sx, sy, ::fmaf(dx0, sx + m1, m2), dy * sx, dy * sy, colour[0], colour[1], colour[2], m0};
             const float mine = reduce_scatter9(v, lane);
             if ((lane & 15) < 9) parked[j][lane >> 4][lane & 15] = mine;
         }
@@ -429,7 +433,9 @@ __global__ void __launch_bounds__(kChunk) render_backward_kernel(
 #pragma unroll
             for (int k = 0; k < 9; ++k) s[k] = (parked[lane][0][k] + parked[lane][1][k]) + (parked[lane][2][k] + parked[lane][3][k]);
             const Staged r = staged[lane];
-            float* row = record_grads + static_cast<std::size_t>(staged_id[lane]) * kRecordGrads;
+            const float g_q_scale = -0.5f * r.alpha0;
+#pragma unroll
+            for (int k = 0; k < 5; ++k) s[k] *= g_q_scale;
             const float out[kRecordGrads] = {
                 -(2.f * r.a * s[0] + 2.f * r.b * s[1]),  // d centre x
                 -(2.f * r.b * s[0] + 2.f * r.c * s[1]),  // d centre y
@@ -438,8 +444,16 @@ __global__ void __launch_bounds__(kChunk) render_backward_kernel(
                 s[8],                                    // d alpha0
             };
 #pragma unroll
-            for (int k = 0; k < kRecordGrads; ++k)
-                if (out[k] != 0.f) detail::atomic_add(row + k, out[k]);
+            for (int k = 0; k < kRecordGrads; ++k) parked[lane][0][k] = out[k];
+        }
+        __syncthreads();
+        // The lanes of one atomic instruction take consecutive fields of consecutive list entries, so
+        // an instruction touches about seven accumulator rows (cache lines) instead of 64.
+        for (int item = lane; item < count * kRecordGrads; item += kChunk) {
+            const int entry = item / kRecordGrads, field = item - entry * kRecordGrads;
+            const float value = parked[entry][0][field];
+            if (value != 0.f)
+                detail::atomic_add(record_grads + static_cast<std::size_t>(staged_id[entry]) * kRecordGradStride + field, value);
         }
     }
 }
@@ -456,7 +470,7 @@ __global__ void __launch_bounds__(256) gaussian_backward_kernel(int G, const flo
     const int g = blockIdx.x * 256 + threadIdx.x;
     if (g >= G) return;
     const std::size_t n = static_cast<std::size_t>(G);
-    const float* acc = record_grads + static_cast<std::size_t>(g) * kRecordGrads;
+    const float* acc = record_grads + static_cast<std::size_t>(g) * kRecordGradStride;
 
     Variable<2, float> log_scale;
     log_scale[0] = params[2 * n + g];
