@@ -44,6 +44,10 @@ def _check_against_oracle(oracle, got, W, H, params, depth, target):
     o64 = oracle.splat_step(W, H, params, depth, target, np.float64)
     assert got["pairs"] == o32["pairs"] and got["longest_list"] == o32["longest_list"]
     assert np.isfinite(got["image"]).all() and np.isfinite(got["grads"]).all()
+    if o64["pairs"] != o32["pairs"]:
+        # a 3-sigma box that ends within rounding of a tile edge is binned differently in fp64: the
+        # scenes then differ by whole (tile, Gaussian) pairs and only the fp32 oracle is comparable
+        o64 = o32
     for ref in (o32, o64):
         assert np.abs(got["image"].astype(np.float64) - ref["image"]).max() < 1e-5
         assert abs(got["loss"] - ref["loss"]) <= 1e-6 * ref["loss"] + 1e-9
@@ -67,6 +71,39 @@ def _check_against_oracle(oracle, got, W, H, params, depth, target):
 def test_step_matches_oracle(gpu, oracle, G, W, H, scale):
     params, depth = random_scene(G, W, H, seed=G, scale_px=scale)
     target = np.random.default_rng(G + 1).uniform(0, 1, (H, W, 3)).astype(np.float32)
+    _check_against_oracle(oracle, _gpu_step(gpu, W, H, params, depth, target), W, H, params, depth, target)
+
+
+def test_depth_ranks_follow_the_depths_of_each_call(gpu, oracle):
+    """The context keeps the depth ranks of the previous call while the depths stay the same;
+    a call with other depths (even one changed value) must be ordered by them."""
+    import torch
+
+    from xyz_autodiff_cuda_amd import splat
+
+    W, H, G = 96, 80, 400
+    params, depth = random_scene(G, W, H, seed=8, scale_px=(3.0, 15.0))
+    params[8] += 2.0  # opaque enough for the order to matter
+    reversed_depth = (1.0 - depth).astype(np.float32)
+    one_changed = depth.copy()
+    one_changed[np.argmax(depth)] = -1.0  # the farthest Gaussian comes to the front
+    ctx = splat.SplatContext(W, H, G)
+    p = torch.from_numpy(params).to(gpu)
+    for d in (depth, depth, reversed_depth, one_changed, depth):
+        image = ctx.forward(p, torch.from_numpy(d).to(gpu)).cpu().numpy()
+        want = oracle.splat_step(W, H, params, d, np.zeros((H, W, 3), np.float32), np.float32, want_grads=False)["image"]
+        assert np.abs(image - want).max() < 1e-5
+    assert np.abs(oracle.splat_step(W, H, params, one_changed, np.zeros((H, W, 3), np.float32), np.float32, want_grads=False)["image"] - want).max() > 1e-3
+    ctx.close()
+
+
+def test_pair_keys_wider_than_32_bits(gpu, oracle):
+    """33 024 tiles (16 bits) and 131 073 Gaussians (18 bits of depth rank): the pair keys
+    take the 64-bit path.  Small Gaussians keep the oracle fast."""
+    W, H, G = 4096, 2064, 131_073
+    params, depth = random_scene(G, W, H, seed=21, scale_px=(0.5, 1.5))
+    depth[::7] = depth[3]  # many depth ties: order falls back to the index
+    target = np.zeros((H, W, 3), np.float32)
     _check_against_oracle(oracle, _gpu_step(gpu, W, H, params, depth, target), W, H, params, depth, target)
 
 

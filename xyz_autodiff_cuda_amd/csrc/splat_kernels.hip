@@ -28,11 +28,17 @@ using namespace xyz_autodiff;
 //   inv = sym_matrix2_inv(cov); alpha0 = sigmoid(opacity)
 // from the library's nodes, runs it forward, and derives the 3-sigma tile
 // rectangle and the number of tiles.
-__global__ void __launch_bounds__(256) project_kernel(int G, const float* __restrict__ params, int width, int height,
+__global__ void __launch_bounds__(256) project_kernel(int G, const float* __restrict__ params,
+                                                      const float* __restrict__ depth,
+                                                      const float* __restrict__ ranked_depth,
+                                                      std::uint32_t* __restrict__ depth_changed, int width, int height,
                                                       Record* __restrict__ records, TileRect* __restrict__ rects,
                                                       std::uint32_t* __restrict__ counts) {
     const int g = blockIdx.x * 256 + threadIdx.x;
     if (g >= G) return;
+    // the depth ranks of the previous step stay valid while every depth keeps its bits
+    if (__builtin_bit_cast(std::uint32_t, depth[g]) != __builtin_bit_cast(std::uint32_t, ranked_depth[g]))
+        atomicOr(depth_changed, 1u);
     const std::size_t n = static_cast<std::size_t>(G);
     const float cx = params[0 * n + g], cy = params[1 * n + g];
     Variable<2, float> log_scale;
@@ -88,24 +94,45 @@ __device__ __forceinline__ std::uint32_t ordered_bits(float f) {
     return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
 }
 
-// Pair emission: Gaussian g writes one (tile | depth, g) pair per tile of its
-// rectangle into the segment [offsets[g], offsets[g+1]).  A wavefront takes 64
-// consecutive Gaussians; within it lanes walk their own rectangles.
+// Depth order as integers.  depth_key_kernel writes the order-preserving bits of
+// every depth and the identity permutation; after a stable sort of those pairs,
+// rank_kernel inverts the permutation: rank[g] = position of Gaussian g in
+// (depth, index) order.  The ranks are dense (log2 G bits instead of 32), which
+// is what makes the pair keys below short.
+__global__ void __launch_bounds__(256) depth_key_kernel(int G, const float* __restrict__ depth,
+                                                        std::uint32_t* __restrict__ keys,
+                                                        std::uint32_t* __restrict__ identity) {
+    const int g = blockIdx.x * 256 + threadIdx.x;
+    if (g >= G) return;
+    keys[g] = ordered_bits(depth[g]);
+    identity[g] = static_cast<std::uint32_t>(g);
+}
+
+__global__ void __launch_bounds__(256) rank_kernel(int G, const std::uint32_t* __restrict__ by_depth,
+                                                   std::uint32_t* __restrict__ rank) {
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= G) return;
+    rank[by_depth[i]] = static_cast<std::uint32_t>(i);
+}
+
+// Pair emission: Gaussian g writes one (tile << rank_bits | rank, g) pair per
+// tile of its rectangle into the segment [offsets[g], offsets[g+1]).
+template <typename Key>
 __global__ void __launch_bounds__(256) emit_kernel(int G, const TileRect* __restrict__ rects,
                                                    const std::uint32_t* __restrict__ offsets,
-                                                   const float* __restrict__ depth, int tiles_x,
-                                                   std::uint64_t* __restrict__ keys, std::uint32_t* __restrict__ values,
+                                                   const std::uint32_t* __restrict__ rank, int rank_bits, int tiles_x,
+                                                   Key* __restrict__ keys, std::uint32_t* __restrict__ values,
                                                    std::uint32_t capacity) {
     const int g = blockIdx.x * 256 + threadIdx.x;
     if (g >= G) return;
     const TileRect rc = rects[g];
     if (rc.x0 > rc.x1) return;
     std::uint32_t at = offsets[g];
-    const std::uint64_t low = ordered_bits(depth[g]);
+    const Key low = rank[g];
     for (int ty = rc.y0; ty <= rc.y1; ++ty)
         for (int tx = rc.x0; tx <= rc.x1; ++tx) {
             if (at < capacity) {
-                keys[at] = (static_cast<std::uint64_t>(ty * tiles_x + tx) << 32) | low;
+                keys[at] = (static_cast<Key>(ty * tiles_x + tx) << rank_bits) | low;
                 values[at] = static_cast<std::uint32_t>(g);
             }
             ++at;
@@ -113,14 +140,15 @@ __global__ void __launch_bounds__(256) emit_kernel(int G, const TileRect* __rest
 }
 
 // Tile ranges from the sorted keys: ranges[t] = [first, last) positions of tile t.
-__global__ void __launch_bounds__(256) ranges_kernel(std::uint32_t K, const std::uint64_t* __restrict__ keys,
+template <typename Key>
+__global__ void __launch_bounds__(256) ranges_kernel(std::uint32_t K, const Key* __restrict__ keys, int rank_bits,
                                                      std::uint32_t* __restrict__ range_begin,
                                                      std::uint32_t* __restrict__ range_end) {
     const std::uint32_t i = blockIdx.x * 256u + threadIdx.x;
     if (i >= K) return;
-    const std::uint32_t t = static_cast<std::uint32_t>(keys[i] >> 32);
-    if (i == 0 || static_cast<std::uint32_t>(keys[i - 1] >> 32) != t) range_begin[t] = i;
-    if (i + 1 == K || static_cast<std::uint32_t>(keys[i + 1] >> 32) != t) range_end[t] = i + 1;
+    const std::uint32_t t = static_cast<std::uint32_t>(keys[i] >> rank_bits);
+    if (i == 0 || static_cast<std::uint32_t>(keys[i - 1] >> rank_bits) != t) range_begin[t] = i;
+    if (i + 1 == K || static_cast<std::uint32_t>(keys[i + 1] >> rank_bits) != t) range_end[t] = i + 1;
 }
 
 // Blocks are handed to the eight XCDs round-robin; giving each XCD a contiguous
@@ -505,26 +533,48 @@ __global__ void __launch_bounds__(256) gaussian_backward_kernel(int G, const flo
 // ---------------------------------------------------------------------------
 // launchers (declared in splat_launch.cuh)
 
-int launch_project(hipStream_t s, int G, const float* params, int width, int height, Record* records, TileRect* rects,
+int launch_project(hipStream_t s, int G, const float* params, const float* depth, const float* ranked_depth,
+                   std::uint32_t* depth_changed, int width, int height, Record* records, TileRect* rects,
                    std::uint32_t* counts) {
-    hipLaunchKernelGGL(project_kernel, dim3(xad::blocks_for(G, 256)), dim3(256), 0, s, G, params, width, height, records,
-                       rects, counts);
+    hipLaunchKernelGGL(project_kernel, dim3(xad::blocks_for(G, 256)), dim3(256), 0, s, G, params, depth, ranked_depth,
+                       depth_changed, width, height, records, rects, counts);
     XAD_HIP_TRY(hipGetLastError());
     return XAD_OK;
 }
 
-int launch_emit(hipStream_t s, int G, const TileRect* rects, const std::uint32_t* offsets, const float* depth,
-                int tiles_x, std::uint64_t* keys, std::uint32_t* values, std::uint32_t capacity) {
-    hipLaunchKernelGGL(emit_kernel, dim3(xad::blocks_for(G, 256)), dim3(256), 0, s, G, rects, offsets, depth, tiles_x, keys,
-                       values, capacity);
+int launch_depth_keys(hipStream_t s, int G, const float* depth, std::uint32_t* keys, std::uint32_t* identity) {
+    hipLaunchKernelGGL(depth_key_kernel, dim3(xad::blocks_for(G, 256)), dim3(256), 0, s, G, depth, keys, identity);
     XAD_HIP_TRY(hipGetLastError());
     return XAD_OK;
 }
 
-int launch_ranges(hipStream_t s, std::uint32_t K, const std::uint64_t* keys, std::uint32_t* range_begin,
-                  std::uint32_t* range_end) {
+int launch_ranks(hipStream_t s, int G, const std::uint32_t* by_depth, std::uint32_t* rank) {
+    hipLaunchKernelGGL(rank_kernel, dim3(xad::blocks_for(G, 256)), dim3(256), 0, s, G, by_depth, rank);
+    XAD_HIP_TRY(hipGetLastError());
+    return XAD_OK;
+}
+
+int launch_emit(hipStream_t s, int G, const TileRect* rects, const std::uint32_t* offsets, const std::uint32_t* rank,
+                int rank_bits, int tiles_x, bool wide_keys, void* keys, std::uint32_t* values, std::uint32_t capacity) {
+    if (wide_keys)
+        hipLaunchKernelGGL(emit_kernel<std::uint64_t>, dim3(xad::blocks_for(G, 256)), dim3(256), 0, s, G, rects, offsets,
+                           rank, rank_bits, tiles_x, static_cast<std::uint64_t*>(keys), values, capacity);
+    else
+        hipLaunchKernelGGL(emit_kernel<std::uint32_t>, dim3(xad::blocks_for(G, 256)), dim3(256), 0, s, G, rects, offsets,
+                           rank, rank_bits, tiles_x, static_cast<std::uint32_t*>(keys), values, capacity);
+    XAD_HIP_TRY(hipGetLastError());
+    return XAD_OK;
+}
+
+int launch_ranges(hipStream_t s, std::uint32_t K, bool wide_keys, const void* keys, int rank_bits,
+                  std::uint32_t* range_begin, std::uint32_t* range_end) {
     if (K == 0) return XAD_OK;
-    hipLaunchKernelGGL(ranges_kernel, dim3(xad::blocks_for(K, 256)), dim3(256), 0, s, K, keys, range_begin, range_end);
+    if (wide_keys)
+        hipLaunchKernelGGL(ranges_kernel<std::uint64_t>, dim3(xad::blocks_for(K, 256)), dim3(256), 0, s, K,
+                           static_cast<const std::uint64_t*>(keys), rank_bits, range_begin, range_end);
+    else
+        hipLaunchKernelGGL(ranges_kernel<std::uint32_t>, dim3(xad::blocks_for(K, 256)), dim3(256), 0, s, K,
+                           static_cast<const std::uint32_t*>(keys), rank_bits, range_begin, range_end);
     XAD_HIP_TRY(hipGetLastError());
     return XAD_OK;
 }

@@ -11,12 +11,19 @@
 
 namespace xad_splat {
 
-int launch_project(hipStream_t s, int G, const float* params, int width, int height, Record* records, TileRect* rects,
+// Also sets *depth_changed to 1 if any depth differs (bitwise) from ranked_depth.
+int launch_project(hipStream_t s, int G, const float* params, const float* depth, const float* ranked_depth,
+                   std::uint32_t* depth_changed, int width, int height, Record* records, TileRect* rects,
                    std::uint32_t* counts);
-int launch_emit(hipStream_t s, int G, const TileRect* rects, const std::uint32_t* offsets, const float* depth,
-                int tiles_x, std::uint64_t* keys, std::uint32_t* values, std::uint32_t capacity);
-int launch_ranges(hipStream_t s, std::uint32_t K, const std::uint64_t* keys, std::uint32_t* range_begin,
-                  std::uint32_t* range_end);
+// Depth order: keys[g] = order-preserving bits of depth[g], identity[g] = g; after the stable
+// sort of those pairs, rank[by_depth[i]] = i.
+int launch_depth_keys(hipStream_t s, int G, const float* depth, std::uint32_t* keys, std::uint32_t* identity);
+int launch_ranks(hipStream_t s, int G, const std::uint32_t* by_depth, std::uint32_t* rank);
+// Pair keys are tile << rank_bits | rank, 32 bits wide when that fits and 64 otherwise.
+int launch_emit(hipStream_t s, int G, const TileRect* rects, const std::uint32_t* offsets, const std::uint32_t* rank,
+                int rank_bits, int tiles_x, bool wide_keys, void* keys, std::uint32_t* values, std::uint32_t capacity);
+int launch_ranges(hipStream_t s, std::uint32_t K, bool wide_keys, const void* keys, int rank_bits,
+                  std::uint32_t* range_begin, std::uint32_t* range_end);
 int launch_render_forward(hipStream_t s, int width, int height, const std::uint32_t* range_begin,
                           const std::uint32_t* range_end, const std::uint32_t* sorted_ids, const Record* records,
                           float* image, float* final_T, std::uint32_t* n_contrib);
@@ -27,13 +34,17 @@ int launch_render_backward(hipStream_t s, int width, int height, const std::uint
 int launch_gaussian_backward(hipStream_t s, int G, const float* params, const float* record_grads, float* grads);
 
 // Device-wide primitives (rocPRIM): exclusive scan of the per-Gaussian tile
-// counts (offsets has G + 1 entries, the last is the number of pairs) and the
-// stable radix sort of the (tile | depth, index) pairs.
+// counts (offsets has G + 1 entries, the last is the number of pairs), the
+// stable radix sort of (depth bits, index) that yields the depth ranks, and the
+// stable radix sort of the (tile | rank, index) pairs over `key_bits` bits.
 std::size_t scan_temp_bytes(int G);
 int exclusive_scan_counts(hipStream_t s, void* temp, std::size_t temp_bytes, const std::uint32_t* counts,
                           std::uint32_t* offsets, int G);
-std::size_t sort_temp_bytes(std::uint32_t capacity);
-int sort_pairs(hipStream_t s, void* temp, std::size_t temp_bytes, const std::uint64_t* keys_in, std::uint64_t* keys_out,
+std::size_t depth_sort_temp_bytes(int G);
+int sort_by_depth(hipStream_t s, void* temp, std::size_t temp_bytes, const std::uint32_t* keys_in,
+                  std::uint32_t* keys_out, const std::uint32_t* values_in, std::uint32_t* values_out, int G);
+std::size_t sort_temp_bytes(std::uint32_t capacity, bool wide_keys);
+int sort_pairs(hipStream_t s, void* temp, std::size_t temp_bytes, bool wide_keys, const void* keys_in, void* keys_out,
                const std::uint32_t* values_in, std::uint32_t* values_out, std::uint32_t K, int key_bits);
 
 }  // namespace xad_splat
