@@ -178,6 +178,7 @@ __device__ __forceinline__ int tile_of_block(int block, int tiles) {
 // (examples/mini-gaussian-splatting/gaussian_splatting_kernel.cu:45-55) in fused form.
 constexpr int kLanePixels = 4;
 constexpr int kChunk = 64;
+constexpr int kPark = 16;  // list entries whose gradient sums are finished and written out together
 constexpr float kHalfLog2e = 0.72134752044448170368f;  // log2(e) / 2
 
 struct alignas(16) Staged {
@@ -242,13 +243,12 @@ __global__ void __launch_bounds__(kChunk) render_forward_kernel(
     const std::uint32_t first = range_begin[tile], last = range_end[tile];
     float T[kLanePixels], red[kLanePixels], green[kLanePixels], blue[kLanePixels];
     std::uint32_t used[kLanePixels];
-    bool done[kLanePixels];
 #pragma unroll
     for (int p = 0; p < kLanePixels; ++p) {
-        T[p] = 1.f;
+        // pixels outside the image start out finished (see below) and are never stored
+        T[p] = (x0 + p < width && y < height) ? 1.f : 0.f;
         red[p] = green[p] = blue[p] = 0.f;
         used[p] = 0;
-        done[p] = !(x0 + p < width && y < height);
     }
 
     for (std::uint32_t base = first; base < last; base += kChunk) {
@@ -265,20 +265,22 @@ __global__ void __launch_bounds__(kChunk) render_forward_kernel(
             const float dx0 = px0 - r.cx;
 #pragma unroll
             for (int p = 0; p < kLanePixels; ++p) {
-                // a pixel stops, for good, before the first Gaussian it meets with T below the threshold
-                done[p] = done[p] || T[p] < kMinTransmittance;
+                // A pixel stops, for good, before the first Gaussian it meets with T below the
+                // threshold: from then on alpha = 0 leaves T where it is, so the test stays true.
+                const bool done = T[p] < kMinTransmittance;
                 const float dx = dx0 + static_cast<float>(p);
                 const float a = math::fp32::exp2_raw(::fmaf(::fmaf(r.a_s, dx, e), dx, f)) * r.alpha0;
-                const float alpha = done[p] ? 0.f : (a > kAlphaMax ? kAlphaMax : a);
+                const float alpha = done ? 0.f : (a > kAlphaMax ? kAlphaMax : a);
                 const float weight = T[p] * alpha;
                 red[p] = ::fmaf(weight, r.red, red[p]);
                 green[p] = ::fmaf(weight, r.green, green[p]);
                 blue[p] = ::fmaf(weight, r.blue, blue[p]);
                 T[p] *= 1.f - alpha;
-                used[p] = done[p] ? used[p] : base - first + j + 1;
+                used[p] = done ? used[p] : base - first + j + 1;
             }
         }
-        const bool all_done = done[0] && done[1] && done[2] && done[3];
+        const bool all_done = T[0] < kMinTransmittance && T[1] < kMinTransmittance && T[2] < kMinTransmittance &&
+                              T[3] < kMinTransmittance;
         if (accumulate::wave::ballot(!all_done) == 0) break;
     }
 #pragma unroll
@@ -353,7 +355,9 @@ __global__ void __launch_bounds__(kChunk) render_backward_kernel(
     double* __restrict__ loss) {
     __shared__ Staged staged[kChunk];
     __shared__ std::uint32_t staged_id[kChunk];
-    __shared__ float parked[kChunk][4][9];  // [list entry][row of 16 lanes][value]
+    // Row sums wait here until a group of kPark list entries is complete.  Small on purpose: LDS per
+    // block, not registers, is what limits the number of resident wavefronts.
+    __shared__ float parked[kPark][4][9];  // [list entry within its group][row of 16 lanes][value]
 
     const int tile = tile_of_block(blockIdx.x, tiles);
     if (tile >= tiles) return;
@@ -409,7 +413,10 @@ __global__ void __launch_bounds__(kChunk) render_backward_kernel(
         }
         __syncthreads();
 
-        for (int j = count - 1; j >= 0; --j) {
+        // groups of up to kPark entries, back to front; all but the last-staged one are full
+        for (int group_end = count; group_end > 0;) {
+        const int group_first = (group_end - 1) / kPark * kPark;
+        for (int j = group_end - 1; j >= group_first; --j) {
             const std::uint32_t position = chunk_first + j;
             const Staged r = staged[j];
             // exponent of the falloff as a polynomial in dx: (a_s dx + e) dx + f
@@ -453,14 +460,15 @@ __global__ void __launch_bounds__(kChunk) render_backward_kernel(
             const float sy = dy * m0;
             const float v[9] = {sx, sy, ::fmaf(dx0, sx + m1, m2), dy * sx, dy * sy, colour[0], colour[1], colour[2], m0};
             const float mine = reduce_scatter9(v, lane);
-            if ((lane & 15) < 9) parked[j][lane >> 4][lane & 15] = mine;
+            if ((lane & 15) < 9) parked[j - group_first][lane >> 4][lane & 15] = mine;
         }
+        const int members = group_end - group_first;
         __syncthreads();
-        if (lane < count) {
+        if (lane < members) {
             float s[9];
 #pragma unroll
             for (int k = 0; k < 9; ++k) s[k] = (parked[lane][0][k] + parked[lane][1][k]) + (parked[lane][2][k] + parked[lane][3][k]);
-            const Staged r = staged[lane];
+            const Staged r = staged[group_first + lane];
             const float g_q_scale = -0.5f * r.alpha0;
 #pragma unroll
             for (int k = 0; k < 5; ++k) s[k] *= g_q_scale;
@@ -477,11 +485,15 @@ __global__ void __launch_bounds__(kChunk) render_backward_kernel(
         __syncthreads();
         // The lanes of one atomic instruction take consecutive fields of consecutive list entries, so
         // an instruction touches about seven accumulator rows (cache lines) instead of 64.
-        for (int item = lane; item < count * kRecordGrads; item += kChunk) {
+        for (int item = lane; item < members * kRecordGrads; item += kChunk) {
             const int entry = item / kRecordGrads, field = item - entry * kRecordGrads;
             const float value = parked[entry][0][field];
             if (value != 0.f)
-                detail::atomic_add(record_grads + static_cast<std::size_t>(staged_id[entry]) * kRecordGradStride + field, value);
+                detail::atomic_add(
+                    record_grads + static_cast<std::size_t>(staged_id[group_first + entry]) * kRecordGradStride + field, value);
+        }
+        __syncthreads();  // the next group parks into the same rows
+        group_end = group_first;
         }
     }
 }
