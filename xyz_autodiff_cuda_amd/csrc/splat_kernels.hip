@@ -270,7 +270,7 @@ __global__ void __launch_bounds__(kChunk) render_forward_kernel(
                 const bool done = T[p] < kMinTransmittance;
                 const float dx = dx0 + static_cast<float>(p);
                 const float a = math::fp32::exp2_raw(::fmaf(::fmaf(r.a_s, dx, e), dx, f)) * r.alpha0;
-                const float alpha = done ? 0.f : (a > kAlphaMax ? kAlphaMax : a);
+                const float alpha = done ? 0.f : __builtin_fminf(a, kAlphaMax);  // a is finite: non-finite Gaussians are not binned
                 const float weight = T[p] * alpha;
                 red[p] = ::fmaf(weight, r.red, red[p]);
                 green[p] = ::fmaf(weight, r.green, green[p]);
@@ -436,7 +436,7 @@ __global__ void __launch_bounds__(kChunk) render_backward_kernel(
                 const float falloff = math::fp32::exp2_raw(::fmaf(::fmaf(r.a_s, dx, e), dx, f));
                 const float a = falloff * r.alpha0;
                 const bool clamped = a > kAlphaMax;
-                const float alpha = active ? (clamped ? kAlphaMax : a) : 0.f;
+                const float alpha = active ? __builtin_fminf(a, kAlphaMax) : 0.f;
                 const float inv = __builtin_amdgcn_rcpf(1.f - alpha);
                 const float T_front = T[p] * inv;  // transmittance in front of this Gaussian
                 const float dot = ::fmaf(dC[p][2], r.blue, ::fmaf(dC[p][1], r.green, dC[p][0] * r.red));
