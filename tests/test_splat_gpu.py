@@ -97,11 +97,12 @@ def test_depth_ranks_follow_the_depths_of_each_call(gpu, oracle):
     ctx.close()
 
 
-def test_pair_keys_wider_than_32_bits(gpu, oracle):
-    """33 024 tiles (16 bits) and 131 073 Gaussians (18 bits of depth rank): the pair keys
-    take the 64-bit path.  Small Gaussians keep the oracle fast."""
-    W, H, G = 4096, 2064, 131_073
+def test_more_than_65536_tiles(gpu, oracle):
+    """256 x 257 tiles: the pair keys (tile indices) take the 32-bit path.  Small Gaussians keep
+    the oracle fast."""
+    W, H, G = 4096, 4112, 60_000
     params, depth = random_scene(G, W, H, seed=21, scale_px=(0.5, 1.5))
+    params[1, :2000] = np.random.default_rng(5).uniform(H - 40, H, 2000)  # populate the last tile rows
     depth[::7] = depth[3]  # many depth ties: order falls back to the index
     target = np.zeros((H, W, 3), np.float32)
     _check_against_oracle(oracle, _gpu_step(gpu, W, H, params, depth, target), W, H, params, depth, target)

@@ -10,9 +10,8 @@ using namespace xad_splat;
 struct xad_splat_context {
     int width = 0, height = 0, G = 0;
     int tiles_x = 0, tiles_y = 0, tiles = 0;
-    int rank_bits = 0;       // bits of a depth rank, ceil(log2 G)
-    int key_bits = 0;        // rank_bits + bits of a tile index
-    bool wide_keys = false;  // pair keys need more than 32 bits
+    int key_bits = 0;        // bits of a tile index: what the pair sort looks at
+    bool wide_keys = false;  // more than 65 536 tiles: 32-bit pair keys instead of 16-bit
     std::uint32_t capacity = 0;  // pairs the workspace can hold
     std::uint32_t pairs = 0;     // pairs of the last step
     bool profile = false;
@@ -22,10 +21,11 @@ struct xad_splat_context {
     std::uint32_t* counts = nullptr;   // G + 1
     std::uint32_t* offsets = nullptr;  // G + 2: exclusive scan of counts, then the depth-changed flag
     std::uint32_t *depth_keys = nullptr, *depth_keys_sorted = nullptr;  // G each
-    std::uint32_t *identity = nullptr, *by_depth = nullptr, *rank = nullptr;  // G each
-    float* ranked_depth = nullptr;  // G: the depths `rank` was computed from
-    bool ranks_valid = false;
-    void *keys = nullptr, *keys_sorted = nullptr;  // 4 or 8 bytes per pair
+    std::uint32_t *identity = nullptr, *by_depth = nullptr;  // G each; by_depth = Gaussians in (depth, index) order
+    float* ranked_depth = nullptr;  // G: the depths by_depth was computed from
+    bool order_valid = false;
+    std::uint32_t* counts_by_depth = nullptr;  // G + 1, the last one stays zero
+    void *keys = nullptr, *keys_sorted = nullptr;  // 2 or 4 bytes per pair
     std::uint32_t *ids = nullptr, *ids_sorted = nullptr;
     std::uint32_t *range_begin = nullptr, *range_end = nullptr;
     float* final_T = nullptr;
@@ -63,7 +63,7 @@ int free_pair_buffers(xad_splat_context* c) {
 int allocate_pair_buffers(xad_splat_context* c, std::uint32_t capacity) {
     free_pair_buffers(c);
     c->capacity = capacity;
-    const std::size_t key_bytes = c->wide_keys ? 8 : 4;
+    const std::size_t key_bytes = c->wide_keys ? 4 : 2;
     XAD_HIP_TRY(hipMalloc(&c->keys, key_bytes * capacity));
     XAD_HIP_TRY(hipMalloc(&c->keys_sorted, key_bytes * capacity));
     XAD_HIP_TRY(hipMalloc(&c->ids, sizeof(std::uint32_t) * capacity));
@@ -77,38 +77,54 @@ void mark(xad_splat_context* c, int index, hipStream_t s) {
     if (c->profile) (void)hipEventRecord(c->marks[index], s);
 }
 
+// (depth, index) order of the Gaussians, kept until a depth changes
+int order_by_depth(xad_splat_context* c, const float* depth, hipStream_t s) {
+    c->order_valid = false;
+    if (int st = launch_depth_keys(s, c->G, depth, c->depth_keys, c->identity)) return st;
+    if (int st = sort_by_depth(s, c->depth_sort_temp, c->depth_sort_bytes, c->depth_keys, c->depth_keys_sorted, c->identity,
+                               c->by_depth, c->G))
+        return st;
+    XAD_HIP_TRY(hipMemcpyAsync(c->ranked_depth, depth, sizeof(float) * c->G, hipMemcpyDeviceToDevice, s));
+    c->order_valid = true;
+    return XAD_OK;
+}
+
+// Places the pairs: scan of the tile counts in depth order.  Reads back the number of pairs
+// (which sizes the sort) and the depth-changed flag: the one synchronisation of a step.
+int place_pairs(xad_splat_context* c, hipStream_t s) {
+    if (int st = launch_permute_counts(s, c->G, c->by_depth, c->counts, c->counts_by_depth)) return st;
+    if (int st = exclusive_scan_counts(s, c->scan_temp, c->scan_bytes, c->counts_by_depth, c->offsets, c->G)) return st;
+    XAD_HIP_TRY(hipMemcpyAsync(c->host_pairs, c->offsets + c->G, 2 * sizeof(std::uint32_t), hipMemcpyDeviceToHost, s));
+    XAD_HIP_TRY(hipStreamSynchronize(s));
+    c->pairs = c->host_pairs[0];
+    return XAD_OK;
+}
+
 // project .. tile ranges; leaves the sorted lists in the context
 int bin(xad_splat_context* c, const float* params, const float* depth, hipStream_t s) {
     mark(c, 0, s);
+    const bool had_order = c->order_valid;
+    if (!had_order)
+        if (int st = order_by_depth(c, depth, s)) return st;
     std::uint32_t* depth_changed = c->offsets + c->G + 1;
     XAD_HIP_TRY(hipMemsetAsync(depth_changed, 0, sizeof(std::uint32_t), s));
     if (int st = launch_project(s, c->G, params, depth, c->ranked_depth, depth_changed, c->width, c->height, c->records,
                                 c->rects, c->counts))
         return st;
     mark(c, 1, s);
-    if (int st = exclusive_scan_counts(s, c->scan_temp, c->scan_bytes, c->counts, c->offsets, c->G)) return st;
-    // the number of pairs sizes the sort; with the depth-changed flag it is all the host has to see
-    XAD_HIP_TRY(hipMemcpyAsync(c->host_pairs, c->offsets + c->G, 2 * sizeof(std::uint32_t), hipMemcpyDeviceToHost, s));
-    XAD_HIP_TRY(hipStreamSynchronize(s));
-    c->pairs = c->host_pairs[0];
-    const bool rerank = !c->ranks_valid || c->host_pairs[1] != 0;
+    // The order of the previous call is used on the assumption that the depths are the same; the
+    // flag read back with the pair count says whether they were, and if not the placement is redone.
+    if (int st = place_pairs(c, s)) return st;
+    if (had_order && c->host_pairs[1] != 0) {
+        if (int st = order_by_depth(c, depth, s)) return st;
+        if (int st = place_pairs(c, s)) return st;
+    }
     if (c->pairs > c->capacity) {
         const std::uint64_t want = static_cast<std::uint64_t>(c->pairs) + c->pairs / 4 + 1024;
         XAD_REQUIRE(want < 0xffffffffull, "splat: %u pairs exceed the 32-bit pair index", c->pairs);
         if (int st = allocate_pair_buffers(c, static_cast<std::uint32_t>(want))) return st;
     }
-    if (rerank) {
-        // depth ranks: (depth, index) order as dense integers; kept until a depth changes
-        c->ranks_valid = false;
-        if (int st = launch_depth_keys(s, c->G, depth, c->depth_keys, c->identity)) return st;
-        if (int st = sort_by_depth(s, c->depth_sort_temp, c->depth_sort_bytes, c->depth_keys, c->depth_keys_sorted,
-                                   c->identity, c->by_depth, c->G))
-            return st;
-        if (int st = launch_ranks(s, c->G, c->by_depth, c->rank)) return st;
-        XAD_HIP_TRY(hipMemcpyAsync(c->ranked_depth, depth, sizeof(float) * c->G, hipMemcpyDeviceToDevice, s));
-        c->ranks_valid = true;
-    }
-    if (int st = launch_emit(s, c->G, c->rects, c->offsets, c->rank, c->rank_bits, c->tiles_x, c->wide_keys, c->keys, c->ids,
+    if (int st = launch_emit(s, c->G, c->by_depth, c->rects, c->offsets, c->tiles_x, c->wide_keys, c->keys, c->ids,
                              c->capacity))
         return st;
     mark(c, 2, s);
@@ -117,8 +133,7 @@ int bin(xad_splat_context* c, const float* params, const float* depth, hipStream
         return st;
     mark(c, 3, s);
     XAD_HIP_TRY(hipMemsetAsync(c->range_begin, 0, sizeof(std::uint32_t) * c->tiles * 2, s));
-    if (int st = launch_ranges(s, c->pairs, c->wide_keys, c->keys_sorted, c->rank_bits, c->range_begin, c->range_end))
-        return st;
+    if (int st = launch_ranges(s, c->pairs, c->wide_keys, c->keys_sorted, c->range_begin, c->range_end)) return st;
     mark(c, 4, s);
     return XAD_OK;
 }
@@ -151,10 +166,8 @@ extern "C" int xad_splat_create(int width, int height, int num_gaussians, std::s
     c->tiles = tiles_x * tiles_y;
     int tile_bits = 1;
     while ((1 << tile_bits) < c->tiles) ++tile_bits;
-    c->rank_bits = 1;
-    while ((1ll << c->rank_bits) < num_gaussians) ++c->rank_bits;
-    c->key_bits = c->rank_bits + tile_bits;
-    c->wide_keys = c->key_bits > 32;
+    c->key_bits = tile_bits;
+    c->wide_keys = c->tiles > 65536;
     const std::size_t pixels = static_cast<std::size_t>(width) * height;
     const std::size_t G = static_cast<std::size_t>(num_gaussians);
     int st = XAD_OK;
@@ -168,7 +181,7 @@ extern "C" int xad_splat_create(int width, int height, int num_gaussians, std::s
     alloc(&c->depth_keys_sorted, sizeof(std::uint32_t) * G);
     alloc(&c->identity, sizeof(std::uint32_t) * G);
     alloc(&c->by_depth, sizeof(std::uint32_t) * G);
-    alloc(&c->rank, sizeof(std::uint32_t) * G);
+    alloc(&c->counts_by_depth, sizeof(std::uint32_t) * (G + 1));
     alloc(&c->counts, sizeof(std::uint32_t) * (G + 1));
     alloc(&c->offsets, sizeof(std::uint32_t) * (G + 2));
     alloc(&c->ranked_depth, sizeof(float) * G);
@@ -190,7 +203,7 @@ extern "C" int xad_splat_create(int width, int height, int num_gaussians, std::s
         st = xad::fail(XAD_ERR_HIP, "%s: pinned allocation failed", who);
     if (st == XAD_OK && hipMemset(c->counts, 0, sizeof(std::uint32_t) * (G + 1)) != hipSuccess)
         st = xad::fail(XAD_ERR_HIP, "%s: hipMemset failed", who);
-    if (st == XAD_OK && hipMemset(c->ranked_depth, 0, sizeof(float) * G) != hipSuccess)
+    if (st == XAD_OK && hipMemset(c->counts_by_depth, 0, sizeof(std::uint32_t) * (G + 1)) != hipSuccess)
         st = xad::fail(XAD_ERR_HIP, "%s: hipMemset failed", who);
     if (st == XAD_OK) {
         const std::size_t hint = pair_capacity_hint ? pair_capacity_hint : G * 8 + 1024;
@@ -215,7 +228,7 @@ extern "C" void xad_splat_destroy(xad_splat_context* c) {
     (void)hipFree(c->depth_keys_sorted);
     (void)hipFree(c->identity);
     (void)hipFree(c->by_depth);
-    (void)hipFree(c->rank);
+    (void)hipFree(c->counts_by_depth);
     (void)hipFree(c->ranked_depth);
     (void)hipFree(c->depth_sort_temp);
     (void)hipFree(c->counts);

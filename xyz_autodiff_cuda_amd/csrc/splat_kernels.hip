@@ -94,11 +94,11 @@ __device__ __forceinline__ std::uint32_t ordered_bits(float f) {
     return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
 }
 
-// Depth order as integers.  depth_key_kernel writes the order-preserving bits of
-// every depth and the identity permutation; after a stable sort of those pairs,
-// rank_kernel inverts the permutation: rank[g] = position of Gaussian g in
-// (depth, index) order.  The ranks are dense (log2 G bits instead of 32), which
-// is what makes the pair keys below short.
+// Depth order.  depth_key_kernel writes the order-preserving bits of every depth
+// and the identity permutation; a stable sort of those pairs gives by_depth, the
+// Gaussians in (depth, index) order.  Pairs are then emitted in that order, so a
+// stable sort on the tile index alone leaves every tile's list in depth order:
+// the pair sort handles 16-bit (or 32-bit) keys instead of tile | depth.
 __global__ void __launch_bounds__(256) depth_key_kernel(int G, const float* __restrict__ depth,
                                                         std::uint32_t* __restrict__ keys,
                                                         std::uint32_t* __restrict__ identity) {
@@ -108,32 +108,34 @@ __global__ void __launch_bounds__(256) depth_key_kernel(int G, const float* __re
     identity[g] = static_cast<std::uint32_t>(g);
 }
 
-__global__ void __launch_bounds__(256) rank_kernel(int G, const std::uint32_t* __restrict__ by_depth,
-                                                   std::uint32_t* __restrict__ rank) {
+// counts in depth order, the input of the scan that places the pairs
+__global__ void __launch_bounds__(256) permute_counts_kernel(int G, const std::uint32_t* __restrict__ by_depth,
+                                                             const std::uint32_t* __restrict__ counts,
+                                                             std::uint32_t* __restrict__ counts_by_depth) {
     const int i = blockIdx.x * 256 + threadIdx.x;
     if (i >= G) return;
-    rank[by_depth[i]] = static_cast<std::uint32_t>(i);
+    counts_by_depth[i] = counts[by_depth[i]];
 }
 
-// Pair emission: Gaussian g writes one (tile << rank_bits | rank, g) pair per
-// tile of its rectangle into the segment [offsets[g], offsets[g+1]).
+// Pair emission: the i-th Gaussian in depth order writes one (tile, index) pair
+// per tile of its rectangle into the segment [offsets[i], offsets[i+1]).
 template <typename Key>
-__global__ void __launch_bounds__(256) emit_kernel(int G, const TileRect* __restrict__ rects,
-                                                   const std::uint32_t* __restrict__ offsets,
-                                                   const std::uint32_t* __restrict__ rank, int rank_bits, int tiles_x,
+__global__ void __launch_bounds__(256) emit_kernel(int G, const std::uint32_t* __restrict__ by_depth,
+                                                   const TileRect* __restrict__ rects,
+                                                   const std::uint32_t* __restrict__ offsets, int tiles_x,
                                                    Key* __restrict__ keys, std::uint32_t* __restrict__ values,
                                                    std::uint32_t capacity) {
-    const int g = blockIdx.x * 256 + threadIdx.x;
-    if (g >= G) return;
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= G) return;
+    const std::uint32_t g = by_depth[i];
     const TileRect rc = rects[g];
     if (rc.x0 > rc.x1) return;
-    std::uint32_t at = offsets[g];
-    const Key low = rank[g];
+    std::uint32_t at = offsets[i];
     for (int ty = rc.y0; ty <= rc.y1; ++ty)
         for (int tx = rc.x0; tx <= rc.x1; ++tx) {
             if (at < capacity) {
-                keys[at] = (static_cast<Key>(ty * tiles_x + tx) << rank_bits) | low;
-                values[at] = static_cast<std::uint32_t>(g);
+                keys[at] = static_cast<Key>(ty * tiles_x + tx);
+                values[at] = g;
             }
             ++at;
         }
@@ -141,14 +143,14 @@ __global__ void __launch_bounds__(256) emit_kernel(int G, const TileRect* __rest
 
 // Tile ranges from the sorted keys: ranges[t] = [first, last) positions of tile t.
 template <typename Key>
-__global__ void __launch_bounds__(256) ranges_kernel(std::uint32_t K, const Key* __restrict__ keys, int rank_bits,
+__global__ void __launch_bounds__(256) ranges_kernel(std::uint32_t K, const Key* __restrict__ keys,
                                                      std::uint32_t* __restrict__ range_begin,
                                                      std::uint32_t* __restrict__ range_end) {
     const std::uint32_t i = blockIdx.x * 256u + threadIdx.x;
     if (i >= K) return;
-    const std::uint32_t t = static_cast<std::uint32_t>(keys[i] >> rank_bits);
-    if (i == 0 || static_cast<std::uint32_t>(keys[i - 1] >> rank_bits) != t) range_begin[t] = i;
-    if (i + 1 == K || static_cast<std::uint32_t>(keys[i + 1] >> rank_bits) != t) range_end[t] = i + 1;
+    const std::uint32_t t = keys[i];
+    if (i == 0 || keys[i - 1] != keys[i]) range_begin[t] = i;
+    if (i + 1 == K || keys[i + 1] != keys[i]) range_end[t] = i + 1;
 }
 
 // Blocks are handed to the eight XCDs round-robin; giving each XCD a contiguous
@@ -560,33 +562,35 @@ int launch_depth_keys(hipStream_t s, int G, const float* depth, std::uint32_t* k
     return XAD_OK;
 }
 
-int launch_ranks(hipStream_t s, int G, const std::uint32_t* by_depth, std::uint32_t* rank) {
-    hipLaunchKernelGGL(rank_kernel, dim3(xad::blocks_for(G, 256)), dim3(256), 0, s, G, by_depth, rank);
+int launch_permute_counts(hipStream_t s, int G, const std::uint32_t* by_depth, const std::uint32_t* counts,
+                          std::uint32_t* counts_by_depth) {
+    hipLaunchKernelGGL(permute_counts_kernel, dim3(xad::blocks_for(G, 256)), dim3(256), 0, s, G, by_depth, counts,
+                       counts_by_depth);
     XAD_HIP_TRY(hipGetLastError());
     return XAD_OK;
 }
 
-int launch_emit(hipStream_t s, int G, const TileRect* rects, const std::uint32_t* offsets, const std::uint32_t* rank,
-                int rank_bits, int tiles_x, bool wide_keys, void* keys, std::uint32_t* values, std::uint32_t capacity) {
+int launch_emit(hipStream_t s, int G, const std::uint32_t* by_depth, const TileRect* rects, const std::uint32_t* offsets,
+                int tiles_x, bool wide_keys, void* keys, std::uint32_t* values, std::uint32_t capacity) {
     if (wide_keys)
-        hipLaunchKernelGGL(emit_kernel<std::uint64_t>, dim3(xad::blocks_for(G, 256)), dim3(256), 0, s, G, rects, offsets,
-                           rank, rank_bits, tiles_x, static_cast<std::uint64_t*>(keys), values, capacity);
+        hipLaunchKernelGGL(emit_kernel<std::uint32_t>, dim3(xad::blocks_for(G, 256)), dim3(256), 0, s, G, by_depth, rects,
+                           offsets, tiles_x, static_cast<std::uint32_t*>(keys), values, capacity);
     else
-        hipLaunchKernelGGL(emit_kernel<std::uint32_t>, dim3(xad::blocks_for(G, 256)), dim3(256), 0, s, G, rects, offsets,
-                           rank, rank_bits, tiles_x, static_cast<std::uint32_t*>(keys), values, capacity);
+        hipLaunchKernelGGL(emit_kernel<std::uint16_t>, dim3(xad::blocks_for(G, 256)), dim3(256), 0, s, G, by_depth, rects,
+                           offsets, tiles_x, static_cast<std::uint16_t*>(keys), values, capacity);
     XAD_HIP_TRY(hipGetLastError());
     return XAD_OK;
 }
 
-int launch_ranges(hipStream_t s, std::uint32_t K, bool wide_keys, const void* keys, int rank_bits,
-                  std::uint32_t* range_begin, std::uint32_t* range_end) {
+int launch_ranges(hipStream_t s, std::uint32_t K, bool wide_keys, const void* keys, std::uint32_t* range_begin,
+                  std::uint32_t* range_end) {
     if (K == 0) return XAD_OK;
     if (wide_keys)
-        hipLaunchKernelGGL(ranges_kernel<std::uint64_t>, dim3(xad::blocks_for(K, 256)), dim3(256), 0, s, K,
-                           static_cast<const std::uint64_t*>(keys), rank_bits, range_begin, range_end);
-    else
         hipLaunchKernelGGL(ranges_kernel<std::uint32_t>, dim3(xad::blocks_for(K, 256)), dim3(256), 0, s, K,
-                           static_cast<const std::uint32_t*>(keys), rank_bits, range_begin, range_end);
+                           static_cast<const std::uint32_t*>(keys), range_begin, range_end);
+    else
+        hipLaunchKernelGGL(ranges_kernel<std::uint16_t>, dim3(xad::blocks_for(K, 256)), dim3(256), 0, s, K,
+                           static_cast<const std::uint16_t*>(keys), range_begin, range_end);
     XAD_HIP_TRY(hipGetLastError());
     return XAD_OK;
 }

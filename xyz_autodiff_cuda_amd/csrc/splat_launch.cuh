@@ -15,15 +15,17 @@ namespace xad_splat {
 int launch_project(hipStream_t s, int G, const float* params, const float* depth, const float* ranked_depth,
                    std::uint32_t* depth_changed, int width, int height, Record* records, TileRect* rects,
                    std::uint32_t* counts);
-// Depth order: keys[g] = order-preserving bits of depth[g], identity[g] = g; after the stable
-// sort of those pairs, rank[by_depth[i]] = i.
+// Depth order: keys[g] = order-preserving bits of depth[g], identity[g] = g; the stable sort of
+// those pairs gives by_depth.  counts_by_depth[i] = counts[by_depth[i]].
 int launch_depth_keys(hipStream_t s, int G, const float* depth, std::uint32_t* keys, std::uint32_t* identity);
-int launch_ranks(hipStream_t s, int G, const std::uint32_t* by_depth, std::uint32_t* rank);
-// Pair keys are tile << rank_bits | rank, 32 bits wide when that fits and 64 otherwise.
-int launch_emit(hipStream_t s, int G, const TileRect* rects, const std::uint32_t* offsets, const std::uint32_t* rank,
-                int rank_bits, int tiles_x, bool wide_keys, void* keys, std::uint32_t* values, std::uint32_t capacity);
-int launch_ranges(hipStream_t s, std::uint32_t K, bool wide_keys, const void* keys, int rank_bits,
-                  std::uint32_t* range_begin, std::uint32_t* range_end);
+int launch_permute_counts(hipStream_t s, int G, const std::uint32_t* by_depth, const std::uint32_t* counts,
+                          std::uint32_t* counts_by_depth);
+// Pairs are emitted in depth order with the tile index as key: 16 bits wide, or 32 (wide_keys)
+// when there are more than 65 536 tiles.
+int launch_emit(hipStream_t s, int G, const std::uint32_t* by_depth, const TileRect* rects, const std::uint32_t* offsets,
+                int tiles_x, bool wide_keys, void* keys, std::uint32_t* values, std::uint32_t capacity);
+int launch_ranges(hipStream_t s, std::uint32_t K, bool wide_keys, const void* keys, std::uint32_t* range_begin,
+                  std::uint32_t* range_end);
 int launch_render_forward(hipStream_t s, int width, int height, const std::uint32_t* range_begin,
                           const std::uint32_t* range_end, const std::uint32_t* sorted_ids, const Record* records,
                           float* image, float* final_T, std::uint32_t* n_contrib);
@@ -35,8 +37,8 @@ int launch_gaussian_backward(hipStream_t s, int G, const float* params, const fl
 
 // Device-wide primitives (rocPRIM): exclusive scan of the per-Gaussian tile
 // counts (offsets has G + 1 entries, the last is the number of pairs), the
-// stable radix sort of (depth bits, index) that yields the depth ranks, and the
-// stable radix sort of the (tile | rank, index) pairs over `key_bits` bits.
+// stable radix sort of (depth bits, index) that yields the depth order, and the
+// stable radix sort of the (tile, index) pairs over the `key_bits` bits of a tile index.
 std::size_t scan_temp_bytes(int G);
 int exclusive_scan_counts(hipStream_t s, void* temp, std::size_t temp_bytes, const std::uint32_t* counts,
                           std::uint32_t* offsets, int G);

@@ -66,14 +66,14 @@ int pair_sort(hipStream_t s, void* temp, std::size_t temp_bytes, const void* key
 }  // namespace
 
 std::size_t sort_temp_bytes(std::uint32_t capacity, bool wide_keys) {
-    return wide_keys ? pair_sort_temp_bytes<std::uint64_t>(capacity) : pair_sort_temp_bytes<std::uint32_t>(capacity);
+    return wide_keys ? pair_sort_temp_bytes<std::uint32_t>(capacity) : pair_sort_temp_bytes<std::uint16_t>(capacity);
 }
 
 int sort_pairs(hipStream_t s, void* temp, std::size_t temp_bytes, bool wide_keys, const void* keys_in, void* keys_out,
                const std::uint32_t* values_in, std::uint32_t* values_out, std::uint32_t K, int key_bits) {
     if (K == 0) return XAD_OK;
-    return wide_keys ? pair_sort<std::uint64_t>(s, temp, temp_bytes, keys_in, keys_out, values_in, values_out, K, key_bits)
-                     : pair_sort<std::uint32_t>(s, temp, temp_bytes, keys_in, keys_out, values_in, values_out, K, key_bits);
+    return wide_keys ? pair_sort<std::uint32_t>(s, temp, temp_bytes, keys_in, keys_out, values_in, values_out, K, key_bits)
+                     : pair_sort<std::uint16_t>(s, temp, temp_bytes, keys_in, keys_out, values_in, values_out, K, key_bits);
 }
 
 }  // namespace xad_splat
