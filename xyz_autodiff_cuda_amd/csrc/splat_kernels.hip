@@ -118,7 +118,12 @@ __global__ void __launch_bounds__(256) permute_counts_kernel(int G, const std::u
 }
 
 // Pair emission: the i-th Gaussian in depth order writes one (tile, index) pair
-// per tile of its rectangle into the segment [offsets[i], offsets[i+1]).
+// per tile of its rectangle into the segment [offsets[i], offsets[i+1]).  A lane
+// writes a small rectangle by itself; a large one (up to hundreds of tiles) is
+// written by its whole wavefront, lane t taking every 64th tile, so the stores
+// are coalesced and no lane is left walking a long rectangle alone.
+constexpr std::uint32_t kEmitAlone = 8;
+
 template <typename Key>
 __global__ void __launch_bounds__(256) emit_kernel(int G, const std::uint32_t* __restrict__ by_depth,
                                                    const TileRect* __restrict__ rects,
@@ -126,19 +131,44 @@ __global__ void __launch_bounds__(256) emit_kernel(int G, const std::uint32_t* _
                                                    Key* __restrict__ keys, std::uint32_t* __restrict__ values,
                                                    std::uint32_t capacity) {
     const int i = blockIdx.x * 256 + threadIdx.x;
-    if (i >= G) return;
-    const std::uint32_t g = by_depth[i];
-    const TileRect rc = rects[g];
-    if (rc.x0 > rc.x1) return;
-    std::uint32_t at = offsets[i];
-    for (int ty = rc.y0; ty <= rc.y1; ++ty)
-        for (int tx = rc.x0; tx <= rc.x1; ++tx) {
-            if (at < capacity) {
-                keys[at] = static_cast<Key>(ty * tiles_x + tx);
-                values[at] = g;
-            }
-            ++at;
+    const int lane = threadIdx.x & 63;
+    std::uint32_t g = 0, at = 0, count = 0;
+    int x0 = 0, y0 = 0, columns = 1;
+    if (i < G) {
+        g = by_depth[i];
+        const TileRect rc = rects[g];
+        if (rc.x0 <= rc.x1) {
+            x0 = rc.x0;
+            y0 = rc.y0;
+            columns = rc.x1 - rc.x0 + 1;
+            count = static_cast<std::uint32_t>(columns) * static_cast<std::uint32_t>(rc.y1 - rc.y0 + 1);
+            at = offsets[i];
         }
+    }
+    if (count <= kEmitAlone) {
+        for (std::uint32_t t = 0; t < count; ++t) {
+            const int ty = y0 + static_cast<int>(t) / columns, tx = x0 + static_cast<int>(t) % columns;
+            if (at + t < capacity) {
+                keys[at + t] = static_cast<Key>(ty * tiles_x + tx);
+                values[at + t] = g;
+            }
+        }
+    }
+    // every lane of the wavefront reaches this loop: the large rectangles are taken one by one
+    for (std::uint64_t large = accumulate::wave::ballot(count > kEmitAlone); large != 0; large &= large - 1) {
+        const int owner = __builtin_ctzll(large);
+        const std::uint32_t n = __builtin_amdgcn_readlane(count, owner), first = __builtin_amdgcn_readlane(at, owner);
+        const std::uint32_t id = __builtin_amdgcn_readlane(g, owner);
+        const int c = __builtin_amdgcn_readlane(columns, owner);
+        const int bx = __builtin_amdgcn_readlane(x0, owner), by = __builtin_amdgcn_readlane(y0, owner);
+        for (std::uint32_t t = lane; t < n; t += 64) {
+            const int ty = by + static_cast<int>(t) / c, tx = bx + static_cast<int>(t) % c;
+            if (first + t < capacity) {
+                keys[first + t] = static_cast<Key>(ty * tiles_x + tx);
+                values[first + t] = id;
+            }
+        }
+    }
 }
 
 // Tile ranges from the sorted keys: ranges[t] = [first, last) positions of tile t.
