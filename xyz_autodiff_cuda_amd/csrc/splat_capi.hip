@@ -9,6 +9,7 @@ using namespace xad_splat;
 
 struct xad_splat_context {
     int width = 0, height = 0, G = 0;
+    int device = 0;  // the device that was current at creation: owns every buffer below
     int tiles_x = 0, tiles_y = 0, tiles = 0;
     int key_bits = 0;        // bits of a tile index: what the pair sort looks at
     bool wide_keys = false;  // more than 65 536 tiles: 32-bit pair keys instead of 16-bit
@@ -62,7 +63,7 @@ int free_pair_buffers(xad_splat_context* c) {
 
 int allocate_pair_buffers(xad_splat_context* c, std::uint32_t capacity) {
     free_pair_buffers(c);
-    c->capacity = capacity;
+    c->capacity = 0;  // stays zero if an allocation below fails: the next call then tries again
     const std::size_t key_bytes = c->wide_keys ? 4 : 2;
     XAD_HIP_TRY(hipMalloc(&c->keys, key_bytes * capacity));
     XAD_HIP_TRY(hipMalloc(&c->keys_sorted, key_bytes * capacity));
@@ -70,6 +71,7 @@ int allocate_pair_buffers(xad_splat_context* c, std::uint32_t capacity) {
     XAD_HIP_TRY(hipMalloc(&c->ids_sorted, sizeof(std::uint32_t) * capacity));
     c->sort_bytes = sort_temp_bytes(capacity, c->wide_keys);
     XAD_HIP_TRY(hipMalloc(&c->sort_temp, c->sort_bytes ? c->sort_bytes : 16));
+    c->capacity = capacity;
     return XAD_OK;
 }
 
@@ -102,6 +104,9 @@ int place_pairs(xad_splat_context* c, hipStream_t s) {
 
 // project .. tile ranges; leaves the sorted lists in the context
 int bin(xad_splat_context* c, const float* params, const float* depth, hipStream_t s) {
+    int current = -1;
+    XAD_HIP_TRY(hipGetDevice(&current));
+    XAD_REQUIRE(current == c->device, "splat: the context belongs to device %d, but device %d is current", c->device, current);
     mark(c, 0, s);
     const bool had_order = c->order_valid;
     if (!had_order)
@@ -161,6 +166,10 @@ extern "C" int xad_splat_create(int width, int height, int num_gaussians, std::s
     c->width = width;
     c->height = height;
     c->G = num_gaussians;
+    if (hipGetDevice(&c->device) != hipSuccess) {
+        delete c;
+        return xad::fail(XAD_ERR_HIP, "%s: no current device", who);
+    }
     c->tiles_x = tiles_x;
     c->tiles_y = tiles_y;
     c->tiles = tiles_x * tiles_y;
