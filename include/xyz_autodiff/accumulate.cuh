@@ -123,14 +123,17 @@ public:
 
     // `lds`: at least lds_bytes(capacity, num_slots > capacity) bytes, 16-byte aligned.
     // `capacity` must be a power of two when num_slots > capacity (tagged mode).
-    // `global`: num_slots x Width values, row-major, already initialised.
+    // `global`: num_slots rows of Width values, already initialised; row s starts at
+    // global + s * row_stride (row_stride = Width for a dense row-major array; a larger
+    // stride lets several accumulators share one array, each owning every k-th row).
     // Clears the table; ends with a block barrier.
-    __device__ BlockAccumulator(void* lds, int capacity, T* global, int num_slots)
+    __device__ BlockAccumulator(void* lds, int capacity, T* global, int num_slots, int row_stride = Width)
         : table_(static_cast<TableT*>(lds)),
           tags_(reinterpret_cast<int*>(static_cast<TableT*>(lds) + static_cast<std::size_t>(capacity) * Width)),
           global_(global),
           capacity_(capacity),
           num_slots_(num_slots),
+          row_stride_(row_stride),
           tagged_(num_slots > capacity),
           shift_(32 - __builtin_ctz(static_cast<unsigned>(capacity))) {
         clear();
@@ -141,7 +144,7 @@ public:
         if constexpr (S == Strategy::GlobalAtomics) {
             if (slot >= 0) {
 #pragma unroll
-                for (int k = 0; k < Width; ++k) detail::atomic_add(global_ + static_cast<std::size_t>(slot) * Width + k, g[k]);
+                for (int k = 0; k < Width; ++k) detail::atomic_add(global_ + static_cast<std::size_t>(slot) * row_stride_ + k, g[k]);
             }
         } else {
             if constexpr (S == Strategy::WaveThenLds) slot = peel(slot, g);
@@ -152,14 +155,14 @@ public:
     // Adds one value to element `element` of slot `slot`.
     __device__ __forceinline__ void add_one(int slot, int element, T value) {
         if constexpr (S == Strategy::GlobalAtomics) {
-            if (slot >= 0) detail::atomic_add(global_ + static_cast<std::size_t>(slot) * Width + element, value);
+            if (slot >= 0) detail::atomic_add(global_ + static_cast<std::size_t>(slot) * row_stride_ + element, value);
         } else {
             if (slot < 0) return;
             const int row = find_row(slot);
             if (row >= 0)
                 detail::atomic_add(table_ + element * capacity_ + row, static_cast<TableT>(value));
             else
-                detail::atomic_add(global_ + static_cast<std::size_t>(slot) * Width + element, value);
+                detail::atomic_add(global_ + static_cast<std::size_t>(slot) * row_stride_ + element, value);
         }
     }
 
@@ -175,7 +178,7 @@ public:
             const int row = e / Width, element = e % Width;
             const int slot = tagged_ ? tags_[row] : row;
             const T v = static_cast<T>(table_[element * capacity_ + row]);
-            if (slot != kEmpty && v != T(0)) detail::atomic_add(global_ + static_cast<std::size_t>(slot) * Width + element, v);
+            if (slot != kEmpty && v != T(0)) detail::atomic_add(global_ + static_cast<std::size_t>(slot) * row_stride_ + element, v);
         }
         __syncthreads();
         clear();
@@ -209,7 +212,7 @@ private:
             for (int k = 0; k < Width; ++k) detail::atomic_add(table_ + k * capacity_ + row, static_cast<TableT>(g[k]));
         } else {
 #pragma unroll
-            for (int k = 0; k < Width; ++k) detail::atomic_add(global_ + static_cast<std::size_t>(slot) * Width + k, g[k]);
+            for (int k = 0; k < Width; ++k) detail::atomic_add(global_ + static_cast<std::size_t>(slot) * row_stride_ + k, g[k]);
         }
     }
 
@@ -244,6 +247,7 @@ private:
     T* global_;
     int capacity_;
     int num_slots_;
+    int row_stride_;
     bool tagged_;
     int shift_;
 };

@@ -59,7 +59,7 @@ def _assert_close(got, ref, sum_tol):
 
 
 @pytest.mark.parametrize("strategy", STAGED)
-@pytest.mark.parametrize("num_slots", [1, 3, 64, 4096, 7000, 262144])
+@pytest.mark.parametrize("num_slots", [1, 3, 64, 3072, 3073, 4096, 5001, 6144, 7000, 262144])
 def test_staged_strategies_match_fp64_sums(gpu, oracle, strategy, num_slots):
     n = 1_000_003
     inputs = chain_inputs(n, seed=50 + num_slots % 97)
@@ -78,13 +78,16 @@ def test_naive_global_atomics(gpu, oracle, strategy, num_slots):
     _assert_close(_run(gpu, inputs, slot, num_slots, strategy), ref, 1e-2)
 
 
-def test_adds_to_existing_values_and_ignores_out_of_range_slots(gpu, oracle):
-    n, num_slots = 100_000, 10
+@pytest.mark.parametrize("num_slots", [10, 5001])  # one table; slots dealt to two tables
+def test_adds_to_existing_values_and_ignores_out_of_range_slots(gpu, oracle, num_slots):
+    n = 100_000
     inputs = chain_inputs(n, seed=3)
     slot = np.random.default_rng(9).integers(-3, num_slots + 3, n).astype(np.int32)
+    slot[::50] = np.random.default_rng(10).choice([-1, -2**31, num_slots, 2**31 - 1], size=slot[::50].size)
     sums, mass, kmass = _reference(oracle, inputs, slot, num_slots)
-    got = _run(gpu, inputs, slot, num_slots, "auto", prefill=2.5)
-    _assert_close(got - 2.5, (sums, mass + 2.5, kmass), 1e-4)
+    for strategy in ("auto", "lds_leaves"):
+        got = _run(gpu, inputs, slot, num_slots, strategy, prefill=2.5)
+        _assert_close(got - 2.5, (sums, mass + 2.5, kmass), 1e-4)
 
 
 def test_uniform_slots_no_contention(gpu, oracle):

@@ -34,24 +34,44 @@ struct AccumulateArgs {
     std::size_t per_block;  // multiple of kBlock
     int num_slots;
     int capacity;
+    // The slots are dealt round-robin to 2^part_shift parts; a block serves one part (blockIdx % parts)
+    // with a table of its own, and the blocks of all parts walk the same threads.  One part = no split.
+    int part_shift;
+};
+
+// Which part a block serves, the rows of its table and where they live in the global array.
+struct Part {
+    int index, parts, rows;
+    __device__ explicit Part(const AccumulateArgs& a)
+        : index(static_cast<int>(blockIdx.x) & ((1 << a.part_shift) - 1)),
+          parts(1 << a.part_shift),
+          rows((a.num_slots - index + parts - 1) >> a.part_shift) {}
+    // table row of slot s, or -1 if s is out of range or belongs to another part
+    __device__ __forceinline__ int row_of(int s, const AccumulateArgs& a) const {
+        const bool mine = static_cast<unsigned>(s) < static_cast<unsigned>(a.num_slots) && (s & (parts - 1)) == index;
+        return mine ? s >> a.part_shift : -1;
+    }
 };
 
 template <Strategy S, int Peel, typename TableT>
 __global__ void __launch_bounds__(kBlock) accumulate_kernel(AccumulateArgs a) {
     extern __shared__ __attribute__((aligned(16))) float lds[];
-    BlockAccumulator<float, kWidth, S, Peel, 4, TableT> acc(lds, a.capacity, a.grads, a.num_slots);
+    const Part part(a);
+    BlockAccumulator<float, kWidth, S, Peel, 4, TableT> acc(lds, a.capacity, a.grads + part.index * kWidth, part.rows,
+                                                            part.parts * kWidth);
 
-    const std::size_t begin = static_cast<std::size_t>(blockIdx.x) * a.per_block;
+    const std::size_t begin = static_cast<std::size_t>(blockIdx.x >> a.part_shift) * a.per_block;
     const std::size_t end = begin + a.per_block < a.n ? begin + a.per_block : a.n;
     for (std::size_t base = begin; base < end; base += kBlock) {
         const std::size_t i = base + threadIdx.x;
         int slot = -1;
         float g[kWidth] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-        if (i < end) {
+        // a slot outside [0, num_slots) is dropped rather than written out of bounds
+        if (i < end) slot = part.row_of(__builtin_nontemporal_load(a.slot + i), a);
+        if (slot >= 0) {
             float x[6];
 #pragma unroll
             for (int k = 0; k < 6; ++k) x[k] = __builtin_nontemporal_load(a.in[k] + i);
-            const int s = __builtin_nontemporal_load(a.slot + i);
             const auto r = xad_chain::forward_backward<float>(x[0], x[1], x[2], x[3], x[4], x[5]);
             g[0] = r.d_sx;
             g[1] = r.d_sy;
@@ -59,8 +79,6 @@ __global__ void __launch_bounds__(kBlock) accumulate_kernel(AccumulateArgs a) {
             g[3] = r.d_o;
             g[4] = r.d_px;
             g[5] = r.d_py;
-            // a slot outside [0, num_slots) is dropped rather than written out of bounds
-            slot = static_cast<unsigned>(s) < static_cast<unsigned>(a.num_slots) ? s : -1;
         }
         acc.add(slot, g);
     }
@@ -75,9 +93,10 @@ __global__ void __launch_bounds__(kBlock) accumulate_leaf_kernel(AccumulateArgs 
     using namespace xyz_autodiff;
     using Acc = BlockAccumulator<float, kWidth, S, 0, 4, TableT>;
     extern __shared__ __attribute__((aligned(16))) float lds[];
-    Acc acc(lds, a.capacity, a.grads, a.num_slots);
+    const Part part(a);
+    Acc acc(lds, a.capacity, a.grads + part.index * kWidth, part.rows, part.parts * kWidth);
 
-    const std::size_t begin = static_cast<std::size_t>(blockIdx.x) * a.per_block;
+    const std::size_t begin = static_cast<std::size_t>(blockIdx.x >> a.part_shift) * a.per_block;
     const std::size_t end = begin + a.per_block < a.n ? begin + a.per_block : a.n;
     for (std::size_t base = begin; base < end; base += kBlock) {
         const std::size_t i = base + threadIdx.x;
@@ -86,8 +105,8 @@ __global__ void __launch_bounds__(kBlock) accumulate_leaf_kernel(AccumulateArgs 
 #pragma unroll
             for (int k = 0; k < 6; ++k) x[k] = __builtin_nontemporal_load(a.in[k] + i);
             const int raw = __builtin_nontemporal_load(a.slot + i);
-            const int slot = static_cast<unsigned>(raw) < static_cast<unsigned>(a.num_slots) ? raw : -1;
-            const float* row = a.grads + static_cast<std::size_t>(slot < 0 ? 0 : slot) * kWidth;
+            const int slot = part.row_of(raw, a);
+            const float* row = a.grads + static_cast<std::size_t>(slot < 0 ? 0 : raw) * kWidth;
             accumulate::SlotRef<2, float, Acc> s(x + 0, acc, slot, 0, row + 0);
             accumulate::SlotRef<1, float, Acc> theta(x + 2, acc, slot, 2, row + 2);
             accumulate::SlotRef<1, float, Acc> opacity(x + 3, acc, slot, 3, row + 3);
@@ -142,11 +161,13 @@ int launch(Kernel kernel, AccumulateArgs a, std::size_t lds_bytes, int blocks_pe
         XAD_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                         static_cast<int>(lds_bytes)));
     const std::size_t chunks = (a.n + kBlock - 1) / kBlock;
-    std::size_t blocks = std::min<std::size_t>(chunks, static_cast<std::size_t>(cus) * blocks_per_cu);
+    const std::size_t resident = std::max<std::size_t>(1, (static_cast<std::size_t>(cus) * blocks_per_cu) >> a.part_shift);
+    std::size_t blocks = std::min<std::size_t>(chunks, resident);  // per part
     const std::size_t chunks_per_block = (chunks + blocks - 1) / blocks;
     a.per_block = chunks_per_block * kBlock;
     blocks = (a.n + a.per_block - 1) / a.per_block;
-    hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(blocks)), dim3(kBlock), lds_bytes, xad::as_stream(stream), a);
+    hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(blocks << a.part_shift)), dim3(kBlock), lds_bytes,
+                       xad::as_stream(stream), a);
     XAD_HIP_TRY(hipGetLastError());
     return XAD_OK;
 }
@@ -159,7 +180,7 @@ extern "C" int xad_accumulate_chain_gradients_f32(int strategy, std::size_t n, c
                                                   void* stream) {
     const char* who = "xad_accumulate_chain_gradients_f32";
     if (n == 0) return XAD_OK;
-    AccumulateArgs a{{sx, sy, theta, o, px, py}, slot, grads, n, 0, num_slots, 0};
+    AccumulateArgs a{{sx, sy, theta, o, px, py}, slot, grads, n, 0, num_slots, 0, 0};
     for (int k = 0; k < 6; ++k) XAD_REQUIRE(a.in[k], "%s: input array %d is null", who, k);
     XAD_REQUIRE(slot && grads, "%s: slot or grads is null", who);
     XAD_REQUIRE(num_slots > 0, "%s: num_slots must be positive, got %d", who, num_slots);
@@ -168,16 +189,23 @@ extern "C" int xad_accumulate_chain_gradients_f32(int strategy, std::size_t n, c
     // wavefront share a slot (measured: a win up to about 8 slots).
     if (strategy == XAD_ACCUMULATE_AUTO) strategy = num_slots <= 8 ? XAD_ACCUMULATE_WAVE_LDS_SHALLOW : XAD_ACCUMULATE_LDS;
 
-    // LDS table (at most 144 KiB): fp64 rows for every slot if they fit; otherwise fp32
-    // rows for every slot if those fit (the slower ds_add_f32 still beats sending the
-    // overflow to HBM); otherwise 4096 fp32 rows claimed on first use.
+    // LDS table (at most 144 KiB): fp64 rows for every slot if they fit; if they fit in two
+    // tables, the slots are dealt to two sets of blocks that each walk all threads (the inputs
+    // are read twice, but ds_add_f64 is that much faster than ds_add_f32); otherwise fp32 rows
+    // for every slot if those fit; otherwise 4096 fp32 rows claimed on first use.
     constexpr std::size_t kTableBudget = 144 * 1024;
-    const std::size_t cells = static_cast<std::size_t>(num_slots) * kWidth;
+    std::size_t cells = static_cast<std::size_t>(num_slots) * kWidth;
     bool f32_table = strategy == XAD_ACCUMULATE_LDS_F32;
+    const bool staged = strategy != XAD_ACCUMULATE_GLOBAL_ATOMICS && strategy != XAD_ACCUMULATE_GLOBAL_LEAVES;
+    if (staged && !f32_table && cells * sizeof(double) > kTableBudget &&
+        ((static_cast<std::size_t>(num_slots) + 1) / 2) * kWidth * sizeof(double) <= kTableBudget) {
+        a.part_shift = 1;
+        cells = ((static_cast<std::size_t>(num_slots) + 1) / 2) * kWidth;
+    }
     if (!f32_table && cells * sizeof(double) > kTableBudget) f32_table = true;
     const std::size_t cell = f32_table ? sizeof(float) : sizeof(double);
     const bool direct = cells * cell <= kTableBudget;
-    a.capacity = direct ? num_slots : 4096;
+    a.capacity = direct ? static_cast<int>(cells / kWidth) : 4096;
     const std::size_t lds = static_cast<std::size_t>(a.capacity) * kWidth * cell + (direct ? 0 : a.capacity * 4u);
     XAD_REQUIRE(lds <= kMaxLdsBytes, "%s: LDS table of %zu bytes does not fit", who, lds);
     const int per_cu = lds <= 32 * 1024 ? 2 : 1;
