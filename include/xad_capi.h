@@ -116,9 +116,10 @@ int xad_host_chain_forward_backward_f64(size_t n,
  *                   block (the reference's shared-memory pattern,
  *                   tests/test_shared_memory_atomic.cu:29-64, made persistent).
  *                   The table is fp64 (ds_add_f64) while num_slots x 6 doubles fit
- *                   in 144 KiB of LDS, else fp32; beyond 6144 slots 4096 fp32 rows
- *                   are claimed on first use and the rest falls through to HBM.
- *                   LDS_F32 forces the fp32 table;
+ *                   in 144 KiB of LDS (3072 slots); up to 6144 slots the slots are
+ *                   dealt to two fp64 tables served by two sets of blocks; beyond
+ *                   that 4096 fp32 rows are claimed on first use and the rest falls
+ *                   through to HBM.  LDS_F32 forces one fp32 table (up to 6144 slots);
  *   WAVE_LDS        DPP pre-reduction of equal slots inside each wavefront (groups
  *                   of >= 4 lanes, up to eight groups per call), then as LDS;
  *                   WAVE_LDS_SHALLOW: at most two groups;
