@@ -108,8 +108,10 @@ __device__ __forceinline__ V sum(V v) {
 }  // namespace wave
 
 template <typename T, int Width, Strategy S = Strategy::LdsAtomics, int PeelRounds = 8, int MinGroup = 4,
-          typename TableT = double>
+          typename TableT = double, bool Spill = false>
 class BlockAccumulator {
+    static_assert(!Spill || sizeof(T) == 4, "spill staging is implemented for 4-byte values");
+
 
 public:
     using table_type = TableT;
@@ -139,6 +141,22 @@ public:
         clear();
     }
 
+    // Bytes of LDS for use_spill_staging() in a block of `threads` lanes.
+    __host__ __device__ static constexpr std::size_t spill_bytes(int threads) {
+        return static_cast<std::size_t>(threads) * (Width + 1) * 4;
+    }
+
+    // With Spill (tagged tables of 4-byte values): contributions that find no row are not sent
+    // to `global` lane by lane (Width instructions, each touching up to 64 rows) but are first
+    // gathered per wavefront in `staging` (spill_bytes(blockDim.x) bytes of LDS, 4-byte aligned)
+    // and written out with consecutive lanes on consecutive elements of consecutive rows, which
+    // cuts the number of memory requests several times.  Must be called before the first add();
+    // add() must then be reached by all lanes of a wavefront together whatever the strategy.
+    __device__ void use_spill_staging(void* staging) {
+        static_assert(Spill, "declare the accumulator with Spill = true");
+        spill_ = static_cast<std::uint32_t*>(staging) + (threadIdx.x / 64) * 64 * (Width + 1);
+    }
+
     // Adds g[0..Width) to slot `slot` (no-op for slot < 0).
     __device__ __forceinline__ void add(int slot, const T (&g)[Width]) {
         if constexpr (S == Strategy::GlobalAtomics) {
@@ -148,7 +166,10 @@ public:
             }
         } else {
             if constexpr (S == Strategy::WaveThenLds) slot = peel(slot, g);
-            if (slot >= 0) deposit(slot, g);
+            if constexpr (Spill)
+                deposit_together(slot, g);
+            else if (slot >= 0)
+                deposit(slot, g);
         }
     }
 
@@ -216,6 +237,38 @@ private:
         }
     }
 
+    // deposit() for a whole wavefront (lanes with slot < 0 have nothing): hits go to the table,
+    // misses are compacted into the wavefront's staging rows (slot, g[0..Width)) and written out
+    // with lane l on element l % Width of staged row l / Width, then the next 64 elements, ...
+    __device__ __forceinline__ void deposit_together(int slot, const T (&g)[Width]) {
+        const int row = slot >= 0 ? find_row(slot) : -1;
+        if (row >= 0) {
+#pragma unroll
+            for (int k = 0; k < Width; ++k) detail::atomic_add(table_ + k * capacity_ + row, static_cast<TableT>(g[k]));
+        }
+        const bool miss = slot >= 0 && row < 0;
+        const std::uint64_t missing = wave::ballot(miss);
+        if (missing == 0) return;
+        if (miss) {
+            const unsigned before = __builtin_amdgcn_mbcnt_hi(static_cast<unsigned>(missing >> 32),
+                                                              __builtin_amdgcn_mbcnt_lo(static_cast<unsigned>(missing), 0u));
+            std::uint32_t* mine = spill_ + before * (Width + 1);
+            mine[0] = static_cast<std::uint32_t>(slot);
+#pragma unroll
+            for (int k = 0; k < Width; ++k) mine[1 + k] = __builtin_bit_cast(std::uint32_t, g[k]);
+        }
+        __builtin_amdgcn_wave_barrier();
+        const int elements = __builtin_popcountll(missing) * Width;
+        for (int e = static_cast<int>(wave::lane_id()); e < elements; e += 64) {
+            const int entry = e / Width, k = e - entry * Width;
+            const std::uint32_t* staged = spill_ + entry * (Width + 1);
+            const T value = __builtin_bit_cast(T, staged[1 + k]);
+            if (value != T(0))
+                detail::atomic_add(global_ + static_cast<std::size_t>(staged[0]) * row_stride_ + k, value);
+        }
+        __builtin_amdgcn_wave_barrier();
+    }
+
     // Level 1.  Take the slot of the first lane that is still waiting and find
     // every lane with the same slot.  If they are at least MinGroup, sum their
     // values across the wavefront, let the first of them deposit the sums, and
@@ -250,6 +303,7 @@ private:
     int row_stride_;
     bool tagged_;
     int shift_;
+    std::uint32_t* spill_ = nullptr;
 };
 
 // A leaf that reads its values like a VariableRef and sends its gradients to a

@@ -37,6 +37,8 @@ struct AccumulateArgs {
     // The slots are dealt round-robin to 2^part_shift parts; a block serves one part (blockIdx % parts)
     // with a table of its own, and the blocks of all parts walk the same threads.  One part = no split.
     int part_shift;
+    // byte offset of the spill staging area in the block's LDS, or 0 for none (tagged tables only)
+    unsigned spill_offset;
 };
 
 // Which part a block serves, the rows of its table and where they live in the global array.
@@ -53,12 +55,13 @@ struct Part {
     }
 };
 
-template <Strategy S, int Peel, typename TableT>
+template <Strategy S, int Peel, typename TableT, bool Spill = false>
 __global__ void __launch_bounds__(kBlock) accumulate_kernel(AccumulateArgs a) {
     extern __shared__ __attribute__((aligned(16))) float lds[];
     const Part part(a);
-    BlockAccumulator<float, kWidth, S, Peel, 4, TableT> acc(lds, a.capacity, a.grads + part.index * kWidth, part.rows,
-                                                            part.parts * kWidth);
+    BlockAccumulator<float, kWidth, S, Peel, 4, TableT, Spill> acc(lds, a.capacity, a.grads + part.index * kWidth,
+                                                                   part.rows, part.parts * kWidth);
+    if constexpr (Spill) acc.use_spill_staging(reinterpret_cast<char*>(lds) + a.spill_offset);
 
     const std::size_t begin = static_cast<std::size_t>(blockIdx.x >> a.part_shift) * a.per_block;
     const std::size_t end = begin + a.per_block < a.n ? begin + a.per_block : a.n;
@@ -180,7 +183,7 @@ extern "C" int xad_accumulate_chain_gradients_f32(int strategy, std::size_t n, c
                                                   void* stream) {
     const char* who = "xad_accumulate_chain_gradients_f32";
     if (n == 0) return XAD_OK;
-    AccumulateArgs a{{sx, sy, theta, o, px, py}, slot, grads, n, 0, num_slots, 0, 0};
+    AccumulateArgs a{{sx, sy, theta, o, px, py}, slot, grads, n, 0, num_slots, 0, 0, 0};
     for (int k = 0; k < 6; ++k) XAD_REQUIRE(a.in[k], "%s: input array %d is null", who, k);
     XAD_REQUIRE(slot && grads, "%s: slot or grads is null", who);
     XAD_REQUIRE(num_slots > 0, "%s: num_slots must be positive, got %d", who, num_slots);
@@ -206,9 +209,24 @@ extern "C" int xad_accumulate_chain_gradients_f32(int strategy, std::size_t n, c
     const std::size_t cell = f32_table ? sizeof(float) : sizeof(double);
     const bool direct = cells * cell <= kTableBudget;
     a.capacity = direct ? static_cast<int>(cells / kWidth) : 4096;
-    const std::size_t lds = static_cast<std::size_t>(a.capacity) * kWidth * cell + (direct ? 0 : a.capacity * 4u);
+    std::size_t lds = static_cast<std::size_t>(a.capacity) * kWidth * cell + (direct ? 0 : a.capacity * 4u);
+    if (!direct && staged && strategy != XAD_ACCUMULATE_LDS_LEAVES) {
+        // slots without a row: gathered per wavefront and written out coalesced
+        a.spill_offset = static_cast<unsigned>(lds);
+        lds += BlockAccumulator<float, kWidth>::spill_bytes(kBlock);
+    }
     XAD_REQUIRE(lds <= kMaxLdsBytes, "%s: LDS table of %zu bytes does not fit", who, lds);
     const int per_cu = lds <= 32 * 1024 ? 2 : 1;
+    if (a.spill_offset) {
+        switch (strategy) {
+            case XAD_ACCUMULATE_WAVE_LDS:
+                return launch(accumulate_kernel<Strategy::WaveThenLds, 8, float, true>, a, lds, per_cu, stream);
+            case XAD_ACCUMULATE_WAVE_LDS_SHALLOW:
+                return launch(accumulate_kernel<Strategy::WaveThenLds, 2, float, true>, a, lds, per_cu, stream);
+            default:
+                return launch(accumulate_kernel<Strategy::LdsAtomics, 0, float, true>, a, lds, per_cu, stream);
+        }
+    }
     if (f32_table && strategy != XAD_ACCUMULATE_GLOBAL_ATOMICS && strategy != XAD_ACCUMULATE_GLOBAL_LEAVES) {
         switch (strategy) {
             case XAD_ACCUMULATE_WAVE_LDS:
