@@ -276,7 +276,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs (profiling runs)")
     ap.add_argument("--counter-probe", choices=("chain", "accumulate", "splat"), default=None,
                     help="launch a few kernels of one leg and exit, for rocprofv3 --pmc runs: chain = a 256 Mi-float "
-                         "copy then three chain passes; accumulate = naive and staged accumulation at 64 and 4096 slots; "
+                         "copy then three chain passes; accumulate = naive and staged accumulation at 64, 4096 and 262144 slots; "
                          "splat = two iterations of the 200k-Gaussian step")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -308,14 +308,14 @@ def main():
 
         m = 16 * 1024 * 1024
         sub = [t[:m] for t in ins]
-        for num_slots in (64, 4096):
+        for num_slots in (64, 4096, 262144):
             slot = torch.empty(m, dtype=torch.int32, device=dev)
             accumulate.zipf_(slot, args.seed, 10, num_slots, 1.1)
             grads = torch.zeros(num_slots, 6, dtype=torch.float32, device=dev)
             for name in ("global_atomics", "auto", "wave_lds"):
                 accumulate.accumulate_chain_gradients(sub, slot, grads, name)
         torch.cuda.synchronize()
-        print(json.dumps({"counter_probe": "accumulate", "n": m, "order": "per slots in (64, 4096): global_atomics, auto, wave_lds"}))
+        print(json.dumps({"counter_probe": "accumulate", "n": m, "order": "per slots in (64, 4096, 262144): global_atomics, auto, wave_lds"}))
         return
     if args.counter_probe == "splat":
         from xyz_autodiff_cuda_amd import splat
