@@ -4,6 +4,22 @@
  * smoke check and the benchmark's CPU-baseline leg compare the HIP path
  * against.  The shipped library never links, loads or calls it.
  *
+ * What pins each part (tests/test_oracle_*.py, tests/test_accumulate_oracle.py);
+ * no function here is left unpinned:
+ *   per-op rules (oracle_ops.inc)  formulas written independently in numpy, central
+ *       differences in fp64, the guards and special cases of the reference's op tests;
+ *   chain (oracle_chain_*)         the reference's own evaluation of the graph at the
+ *       points of tests/golden/chain_reference_vector.json, a closed form without a
+ *       matrix inverse, central differences;
+ *   accumulation sums              a bincount formulation and the reference's exact
+ *       counting pattern (tests/test_parallel_gradient_accumulation.cu:94-99);
+ *   least squares (oracle_linreg.c) hand-computed gradients at the reference's test
+ *       points, a closed form, central differences, one-step and schedule closed forms;
+ *   Adam (oracle_adam.c) and the renderer (oracle_splat.inc): the reference's tests
+ *       hold no expected values for either (parity with the reference is unpinned
+ *       in that sense); pinned by closed forms, an fp64 recurrence, a brute-force
+ *       renderer, invariance to listing order and central differences of the loss.
+ *
  * Built twice over by the preprocessor: every op exists as name_f32 (float
  * arithmetic with the float libm routines, i.e. what the reference computes in
  * device code) and name_f64 (double).  Compile with contraction off so each
