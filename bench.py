@@ -22,7 +22,7 @@ if ROOT not in sys.path:
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published
 # HBM bytes per evaluation of the chain kernel, from FETCH_SIZE / WRITE_SIZE counter
 # passes scaled by a copy of known size (profiles/chain_single_kernel_hbm_traffic.md)
-MEASURED_TRAFFIC_BYTES_PER_EVAL = 52.003
+MEASURED_TRAFFIC_BYTES_PER_EVAL = 52.001
 N_FULL = 64 * 1024 * 1024
 
 

@@ -10,10 +10,14 @@
 //   - one problem per lane, 4-byte accesses, 512-lane blocks: each wavefront
 //     instruction covers 256 contiguous bytes of one array and a block covers
 //     2 KiB of each.  This is the faster one on MI355X for 13 concurrent streams
-//     (measured ~6.3 TB/s against ~5.7 TB/s) and the default;
+//     (measured ~5.9 TB/s against ~5.0 TB/s) and the default;
 //   - four consecutive problems per lane, 16-byte accesses (1 KiB per wavefront
 //     instruction), selectable for comparison.
-// All accesses are marked non-temporal: nothing is reused.
+// Loads are marked non-temporal (nothing is reused).  Stores of the default
+// kernel are ordinary ones: measured over 16 alternating trials on two
+// machines, 5.91-5.92 TB/s against 5.80-5.81 TB/s with non-temporal stores (and
+// 5.67 TB/s with ordinary loads as well); the stream-copy yardstick and the
+// 16-byte kernel keep non-temporal stores.
 #include <algorithm>
 #include <thread>
 #include <vector>
@@ -61,7 +65,7 @@ __global__ void __launch_bounds__(kQuadBlock) chain_quad_kernel(ChainBuffers buf
     for (int a = 0; a < 7; ++a) store4_stream(buf.out[a], g, out[a]);
 }
 
-// One lane, one problem, 4-byte accesses; problems first .. n-1.
+// One lane, one problem, 4-byte accesses; problems first .. n-1.  Non-temporal loads, ordinary stores.
 __global__ void __launch_bounds__(kSingleBlock) chain_single_kernel(ChainBuffers buf, std::size_t first, std::size_t n) {
     const std::size_t i = first + static_cast<std::size_t>(blockIdx.x) * kSingleBlock + threadIdx.x;
     if (i >= n) return;
@@ -71,7 +75,7 @@ __global__ void __launch_bounds__(kSingleBlock) chain_single_kernel(ChainBuffers
     const auto r = xad_chain::forward_backward<float>(x[0], x[1], x[2], x[3], x[4], x[5]);
     const float y[7] = {r.w, r.d_sx, r.d_sy, r.d_theta, r.d_o, r.d_px, r.d_py};
 #pragma unroll
-    for (int a = 0; a < 7; ++a) __builtin_nontemporal_store(y[a], buf.out[a] + i);
+    for (int a = 0; a < 7; ++a) buf.out[a][i] = y[a];
 }
 
 // Plain copy with the chain kernel's access pattern (4 bytes per lane, non-temporal):
