@@ -111,12 +111,14 @@ int xad_host_chain_forward_backward_f64(size_t n,
  *   GLOBAL_ATOMICS  one global atomic per thread per element: the pattern of
  *                   VariableRef::add_grad (include/xyz_autodiff/variable.cuh:48-50;
  *                   tests/test_parallel_gradient_accumulation.cu:25-49);
- *   AUTO            WAVE_LDS_SHALLOW for num_slots <= 8, LDS otherwise (the measured optimum);
+ *   AUTO            LDS (the measured optimum at every slot count from 1 to 262 144);
  *   LDS             per-block table of partial sums in LDS, written out once per
  *                   block (the reference's shared-memory pattern,
  *                   tests/test_shared_memory_atomic.cu:29-64, made persistent).
  *                   The table is fp64 (ds_add_f64) while num_slots x 6 doubles fit
- *                   in 144 KiB of LDS (3072 slots); up to 6144 slots the slots are
+ *                   in 144 KiB of LDS (3072 slots), kept in up to 16 copies while
+ *                   those fit in 48 KiB so that lanes sharing a slot do not share an
+ *                   address; up to 6144 slots the slots are
  *                   dealt to two fp64 tables served by two sets of blocks; beyond
  *                   that 4096 fp32 rows are claimed on first use and the rest falls
  *                   through to HBM.  LDS_F32 forces one fp32 table (up to 6144 slots);

@@ -22,10 +22,12 @@
 // whatever its addresses (3 cycles per lane), a ds_add_f64 for 8 cycles when
 // the 64 addresses are distinct, plus about 3 cycles per lane that shares an
 // address with another.  So partial sums are kept in fp64 (which also makes them
-// more accurate than the fp32 running sums of plain atomics), and level 1 exists
-// to take the lanes that share a slot out of the LDS instruction: summing a
-// group of m lanes costs about 60 VALU issue cycles once and saves about
-// 3 m Width LDS cycles, which pays from m = 4 on (MinGroup).
+// more accurate than the fp32 running sums of plain atomics).  Two ways to take
+// the sharing lanes out of the LDS instruction: a small table can be replicated,
+// lane l adding into copy l % replicas (no extra instructions; the fastest at
+// every slot count measured), or level 1 can sum a group of m sharing lanes
+// first, which costs about 60 VALU issue cycles per group and saves about
+// 3 m Width LDS cycles (MinGroup = 4 is where that starts to pay).
 //
 // The LDS table holds `capacity` slots of Width values, stored element-major
 // (all slots' element 0, then element 1, ...) so that the lanes of one
@@ -128,18 +130,29 @@ public:
     // `global`: num_slots rows of Width values, already initialised; row s starts at
     // global + s * row_stride (row_stride = Width for a dense row-major array; a larger
     // stride lets several accumulators share one array, each owning every k-th row).
+    // `replicas` (a power of two; 1 = none): a small table is kept that many times and lane l
+    // adds into copy l % replicas, so lanes of one instruction that share a slot no longer
+    // share an address (each sharing lane costs an LDS atomic about 3 cycles); flush() adds the
+    // copies up.  Needs capacity >= replica_rows(num_slots) * replicas.
     // Clears the table; ends with a block barrier.
-    __device__ BlockAccumulator(void* lds, int capacity, T* global, int num_slots, int row_stride = Width)
+    __device__ BlockAccumulator(void* lds, int capacity, T* global, int num_slots, int row_stride = Width,
+                                int replicas = 1)
         : table_(static_cast<TableT*>(lds)),
           tags_(reinterpret_cast<int*>(static_cast<TableT*>(lds) + static_cast<std::size_t>(capacity) * Width)),
           global_(global),
           capacity_(capacity),
           num_slots_(num_slots),
           row_stride_(row_stride),
-          tagged_(num_slots > capacity),
-          shift_(32 - __builtin_ctz(static_cast<unsigned>(capacity))) {
+          tagged_(replicas == 1 && num_slots > capacity),
+          shift_(32 - __builtin_ctz(static_cast<unsigned>(capacity))),
+          replicas_(replicas),
+          my_copy_(static_cast<int>(wave::lane_id() & static_cast<unsigned>(replicas - 1)) * replica_rows(num_slots)) {
         clear();
     }
+
+    // Rows one copy of a replicated table occupies: odd, so that the copies of a slot fall
+    // into different LDS banks.
+    __host__ __device__ static constexpr int replica_rows(int num_slots) { return num_slots | 1; }
 
     // Bytes of LDS for use_spill_staging() in a block of `threads` lanes.
     __host__ __device__ static constexpr std::size_t spill_bytes(int threads) {
@@ -195,10 +208,13 @@ public:
         // e runs over the global layout (slot-major) so the atomics of a
         // wavefront touch consecutive addresses.
         const int rows = tagged_ ? capacity_ : num_slots_;
+        const int copy_rows = replica_rows(num_slots_);
         for (int e = threadIdx.x; e < rows * Width; e += blockDim.x) {
             const int row = e / Width, element = e % Width;
             const int slot = tagged_ ? tags_[row] : row;
-            const T v = static_cast<T>(table_[element * capacity_ + row]);
+            TableT sum = table_[element * capacity_ + row];
+            for (int copy = 1; copy < replicas_; ++copy) sum += table_[element * capacity_ + copy * copy_rows + row];
+            const T v = static_cast<T>(sum);
             if (slot != kEmpty && v != T(0)) detail::atomic_add(global_ + static_cast<std::size_t>(slot) * row_stride_ + element, v);
         }
         __syncthreads();
@@ -216,7 +232,7 @@ private:
 
     // Row of the LDS table that holds `slot`, or -1 if the slot has none.
     __device__ __forceinline__ int find_row(int slot) {
-        if (!tagged_) return slot;
+        if (!tagged_) return slot + my_copy_;
         const int row = static_cast<int>((static_cast<unsigned>(slot) * 2654435761u) >> shift_);
         int owner = tags_[row];
         if (owner == kEmpty) {
@@ -303,6 +319,8 @@ private:
     int row_stride_;
     bool tagged_;
     int shift_;
+    int replicas_;
+    int my_copy_;  // first row of this lane's copy of the table
     std::uint32_t* spill_ = nullptr;
 };
 

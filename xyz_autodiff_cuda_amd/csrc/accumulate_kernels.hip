@@ -39,6 +39,8 @@ struct AccumulateArgs {
     int part_shift;
     // byte offset of the spill staging area in the block's LDS, or 0 for none (tagged tables only)
     unsigned spill_offset;
+    // copies of a small table, so that lanes sharing a slot do not share an LDS address
+    int replicas;
 };
 
 // Which part a block serves, the rows of its table and where they live in the global array.
@@ -60,7 +62,7 @@ __global__ void __launch_bounds__(kBlock) accumulate_kernel(AccumulateArgs a) {
     extern __shared__ __attribute__((aligned(16))) float lds[];
     const Part part(a);
     BlockAccumulator<float, kWidth, S, Peel, 4, TableT, Spill> acc(lds, a.capacity, a.grads + part.index * kWidth,
-                                                                   part.rows, part.parts * kWidth);
+                                                                   part.rows, part.parts * kWidth, a.replicas);
     if constexpr (Spill) acc.use_spill_staging(reinterpret_cast<char*>(lds) + a.spill_offset);
 
     const std::size_t begin = static_cast<std::size_t>(blockIdx.x >> a.part_shift) * a.per_block;
@@ -97,7 +99,7 @@ __global__ void __launch_bounds__(kBlock) accumulate_leaf_kernel(AccumulateArgs 
     using Acc = BlockAccumulator<float, kWidth, S, 0, 4, TableT>;
     extern __shared__ __attribute__((aligned(16))) float lds[];
     const Part part(a);
-    Acc acc(lds, a.capacity, a.grads + part.index * kWidth, part.rows, part.parts * kWidth);
+    Acc acc(lds, a.capacity, a.grads + part.index * kWidth, part.rows, part.parts * kWidth, a.replicas);
 
     const std::size_t begin = static_cast<std::size_t>(blockIdx.x >> a.part_shift) * a.per_block;
     const std::size_t end = begin + a.per_block < a.n ? begin + a.per_block : a.n;
@@ -183,14 +185,14 @@ extern "C" int xad_accumulate_chain_gradients_f32(int strategy, std::size_t n, c
                                                   void* stream) {
     const char* who = "xad_accumulate_chain_gradients_f32";
     if (n == 0) return XAD_OK;
-    AccumulateArgs a{{sx, sy, theta, o, px, py}, slot, grads, n, 0, num_slots, 0, 0, 0};
+    AccumulateArgs a{{sx, sy, theta, o, px, py}, slot, grads, n, 0, num_slots, 0, 0, 0, 1};
     for (int k = 0; k < 6; ++k) XAD_REQUIRE(a.in[k], "%s: input array %d is null", who, k);
     XAD_REQUIRE(slot && grads, "%s: slot or grads is null", who);
     XAD_REQUIRE(num_slots > 0, "%s: num_slots must be positive, got %d", who, num_slots);
 
-    // Strategy AUTO: wavefront pre-reduction only pays when nearly all lanes of a
-    // wavefront share a slot (measured: a win up to about 8 slots).
-    if (strategy == XAD_ACCUMULATE_AUTO) strategy = num_slots <= 8 ? XAD_ACCUMULATE_WAVE_LDS_SHALLOW : XAD_ACCUMULATE_LDS;
+    // Strategy AUTO: the LDS table.  With small tables replicated (below) it is the fastest at every
+    // slot count measured, 1 to 262 144; the wavefront pre-reduction stays selectable.
+    if (strategy == XAD_ACCUMULATE_AUTO) strategy = XAD_ACCUMULATE_LDS;
 
     // LDS table (at most 144 KiB): fp64 rows for every slot if they fit; if they fit in two
     // tables, the slots are dealt to two sets of blocks that each walk all threads (the inputs
@@ -209,7 +211,14 @@ extern "C" int xad_accumulate_chain_gradients_f32(int strategy, std::size_t n, c
     const std::size_t cell = f32_table ? sizeof(float) : sizeof(double);
     const bool direct = cells * cell <= kTableBudget;
     a.capacity = direct ? static_cast<int>(cells / kWidth) : 4096;
+    if (direct && staged && a.part_shift == 0) {
+        // a small table is replicated: up to 16 copies within 48 KiB (two blocks per CU stay resident)
+        const std::size_t copy_rows = static_cast<std::size_t>(BlockAccumulator<float, kWidth>::replica_rows(num_slots));
+        while (a.replicas < 16 && copy_rows * (a.replicas * 2) * kWidth * cell <= 48 * 1024) a.replicas *= 2;
+        if (a.replicas > 1) a.capacity = static_cast<int>(copy_rows) * a.replicas;
+    }
     std::size_t lds = static_cast<std::size_t>(a.capacity) * kWidth * cell + (direct ? 0 : a.capacity * 4u);
+    if (lds < 16) lds = 16;
     if (!direct && staged && strategy != XAD_ACCUMULATE_LDS_LEAVES) {
         // slots without a row: gathered per wavefront and written out coalesced
         a.spill_offset = static_cast<unsigned>(lds);
