@@ -164,9 +164,12 @@ int xad_accumulate_chain_gradients_f32(int strategy, size_t n,
  *
  * The context owns all intermediate device buffers (records, pair lists, sort
  * workspace, per-pixel state); they grow when a step produces more (tile,
- * Gaussian) pairs than fit.  A step reads one 4-byte count back to size the
- * sort, so calls synchronise with `stream` once.  One context serves one stream
- * at a time.
+ * Gaussian) pairs than fit.  A step reads two words back (the pair count, which
+ * sizes the sort, and whether any depth differs from the previous call's), so
+ * calls synchronise with `stream` once; the order of the Gaussians by (depth,
+ * index) is kept between calls and recomputed, with one more synchronisation,
+ * only in a call whose depths differ.  One context serves one stream at a time
+ * and belongs to the device that was current when it was created.
  */
 typedef struct xad_splat_context xad_splat_context;
 int xad_splat_create(int width, int height, int num_gaussians, size_t pair_capacity_hint,

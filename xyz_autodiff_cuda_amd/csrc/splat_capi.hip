@@ -23,7 +23,7 @@ struct xad_splat_context {
     std::uint32_t* offsets = nullptr;  // G + 2: exclusive scan of counts, then the depth-changed flag
     std::uint32_t *depth_keys = nullptr, *depth_keys_sorted = nullptr;  // G each
     std::uint32_t *identity = nullptr, *by_depth = nullptr;  // G each; by_depth = Gaussians in (depth, index) order
-    float* ranked_depth = nullptr;  // G: the depths by_depth was computed from
+    float* ordered_depth = nullptr;  // G: the depths by_depth was computed from
     bool order_valid = false;
     std::uint32_t* counts_by_depth = nullptr;  // G + 1, the last one stays zero
     void *keys = nullptr, *keys_sorted = nullptr;  // 2 or 4 bytes per pair
@@ -86,7 +86,7 @@ int order_by_depth(xad_splat_context* c, const float* depth, hipStream_t s) {
     if (int st = sort_by_depth(s, c->depth_sort_temp, c->depth_sort_bytes, c->depth_keys, c->depth_keys_sorted, c->identity,
                                c->by_depth, c->G))
         return st;
-    XAD_HIP_TRY(hipMemcpyAsync(c->ranked_depth, depth, sizeof(float) * c->G, hipMemcpyDeviceToDevice, s));
+    XAD_HIP_TRY(hipMemcpyAsync(c->ordered_depth, depth, sizeof(float) * c->G, hipMemcpyDeviceToDevice, s));
     c->order_valid = true;
     return XAD_OK;
 }
@@ -113,7 +113,7 @@ int bin(xad_splat_context* c, const float* params, const float* depth, hipStream
         if (int st = order_by_depth(c, depth, s)) return st;
     std::uint32_t* depth_changed = c->offsets + c->G + 1;
     XAD_HIP_TRY(hipMemsetAsync(depth_changed, 0, sizeof(std::uint32_t), s));
-    if (int st = launch_project(s, c->G, params, depth, c->ranked_depth, depth_changed, c->width, c->height, c->records,
+    if (int st = launch_project(s, c->G, params, depth, c->ordered_depth, depth_changed, c->width, c->height, c->records,
                                 c->rects, c->counts))
         return st;
     mark(c, 1, s);
@@ -193,7 +193,7 @@ extern "C" int xad_splat_create(int width, int height, int num_gaussians, std::s
     alloc(&c->counts_by_depth, sizeof(std::uint32_t) * (G + 1));
     alloc(&c->counts, sizeof(std::uint32_t) * (G + 1));
     alloc(&c->offsets, sizeof(std::uint32_t) * (G + 2));
-    alloc(&c->ranked_depth, sizeof(float) * G);
+    alloc(&c->ordered_depth, sizeof(float) * G);
     alloc(&c->range_begin, sizeof(std::uint32_t) * c->tiles * 2);
     alloc(&c->final_T, sizeof(float) * pixels);
     alloc(&c->n_contrib, sizeof(std::uint32_t) * pixels);
@@ -238,7 +238,7 @@ extern "C" void xad_splat_destroy(xad_splat_context* c) {
     (void)hipFree(c->identity);
     (void)hipFree(c->by_depth);
     (void)hipFree(c->counts_by_depth);
-    (void)hipFree(c->ranked_depth);
+    (void)hipFree(c->ordered_depth);
     (void)hipFree(c->depth_sort_temp);
     (void)hipFree(c->counts);
     (void)hipFree(c->offsets);

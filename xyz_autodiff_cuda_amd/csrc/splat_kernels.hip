@@ -30,14 +30,14 @@ using namespace xyz_autodiff;
 // rectangle and the number of tiles.
 __global__ void __launch_bounds__(256) project_kernel(int G, const float* __restrict__ params,
                                                       const float* __restrict__ depth,
-                                                      const float* __restrict__ ranked_depth,
+                                                      const float* __restrict__ ordered_depth,
                                                       std::uint32_t* __restrict__ depth_changed, int width, int height,
                                                       Record* __restrict__ records, TileRect* __restrict__ rects,
                                                       std::uint32_t* __restrict__ counts) {
     const int g = blockIdx.x * 256 + threadIdx.x;
     if (g >= G) return;
-    // the depth ranks of the previous step stay valid while every depth keeps its bits
-    if (__builtin_bit_cast(std::uint32_t, depth[g]) != __builtin_bit_cast(std::uint32_t, ranked_depth[g]))
+    // the depth order of the previous call stays valid while every depth keeps its bits
+    if (__builtin_bit_cast(std::uint32_t, depth[g]) != __builtin_bit_cast(std::uint32_t, ordered_depth[g]))
         atomicOr(depth_changed, 1u);
     const std::size_t n = static_cast<std::size_t>(G);
     const float cx = params[0 * n + g], cy = params[1 * n + g];
@@ -577,10 +577,10 @@ __global__ void __launch_bounds__(256) gaussian_backward_kernel(int G, const flo
 // ---------------------------------------------------------------------------
 // launchers (declared in splat_launch.cuh)
 
-int launch_project(hipStream_t s, int G, const float* params, const float* depth, const float* ranked_depth,
+int launch_project(hipStream_t s, int G, const float* params, const float* depth, const float* ordered_depth,
                    std::uint32_t* depth_changed, int width, int height, Record* records, TileRect* rects,
                    std::uint32_t* counts) {
-    hipLaunchKernelGGL(project_kernel, dim3(xad::blocks_for(G, 256)), dim3(256), 0, s, G, params, depth, ranked_depth,
+    hipLaunchKernelGGL(project_kernel, dim3(xad::blocks_for(G, 256)), dim3(256), 0, s, G, params, depth, ordered_depth,
                        depth_changed, width, height, records, rects, counts);
     XAD_HIP_TRY(hipGetLastError());
     return XAD_OK;

@@ -11,8 +11,8 @@
 
 namespace xad_splat {
 
-// Also sets *depth_changed to 1 if any depth differs (bitwise) from ranked_depth.
-int launch_project(hipStream_t s, int G, const float* params, const float* depth, const float* ranked_depth,
+// Also sets *depth_changed to 1 if any depth differs (bitwise) from ordered_depth.
+int launch_project(hipStream_t s, int G, const float* params, const float* depth, const float* ordered_depth,
                    std::uint32_t* depth_changed, int width, int height, Record* records, TileRect* rects,
                    std::uint32_t* counts);
 // Depth order: keys[g] = order-preserving bits of depth[g], identity[g] = g; the stable sort of
