@@ -14,10 +14,13 @@
 //   - four consecutive problems per lane, 16-byte accesses (1 KiB per wavefront
 //     instruction), selectable for comparison.
 // Loads are marked non-temporal (nothing is reused).  Stores of the default
-// kernel are ordinary ones: measured over 16 alternating trials on two
-// machines, 5.91-5.92 TB/s against 5.80-5.81 TB/s with non-temporal stores (and
-// 5.67 TB/s with ordinary loads as well); the stream-copy yardstick and the
-// 16-byte kernel keep non-temporal stores.
+// kernel are relaxed atomic stores at agent scope, which on gfx950 are ordinary
+// 4-byte stores with the sc1 cache-policy bit (written through the L2 instead of
+// being held there).  Measured in alternating trials of the same kernel body:
+// 6.18-6.20 TB/s, against 5.91-5.92 with plain stores, 5.80-5.81 with
+// non-temporal stores, 5.99-6.04 with sc1 and nt together, and 5.67 with plain
+// loads and stores; the stream-copy yardstick and the 16-byte kernel keep
+// non-temporal stores.
 #include <algorithm>
 #include <thread>
 #include <vector>
@@ -65,7 +68,7 @@ __global__ void __launch_bounds__(kQuadBlock) chain_quad_kernel(ChainBuffers buf
     for (int a = 0; a < 7; ++a) store4_stream(buf.out[a], g, out[a]);
 }
 
-// One lane, one problem, 4-byte accesses; problems first .. n-1.  Non-temporal loads, ordinary stores.
+// One lane, one problem, 4-byte accesses; problems first .. n-1.  Non-temporal loads, write-through stores.
 __global__ void __launch_bounds__(kSingleBlock) chain_single_kernel(ChainBuffers buf, std::size_t first, std::size_t n) {
     const std::size_t i = first + static_cast<std::size_t>(blockIdx.x) * kSingleBlock + threadIdx.x;
     if (i >= n) return;
@@ -75,7 +78,7 @@ __global__ void __launch_bounds__(kSingleBlock) chain_single_kernel(ChainBuffers
     const auto r = xad_chain::forward_backward<float>(x[0], x[1], x[2], x[3], x[4], x[5]);
     const float y[7] = {r.w, r.d_sx, r.d_sy, r.d_theta, r.d_o, r.d_px, r.d_py};
 #pragma unroll
-    for (int a = 0; a < 7; ++a) buf.out[a][i] = y[a];
+    for (int a = 0; a < 7; ++a) __hip_atomic_store(buf.out[a] + i, y[a], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // Plain copy with the chain kernel's access pattern (4 bytes per lane, non-temporal):
