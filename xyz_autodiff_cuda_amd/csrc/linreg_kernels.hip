@@ -75,22 +75,39 @@ __global__ void __launch_bounds__(kBlock) linreg_leaf_kernel(LinregArgs a) {
 // Register leaves: each lane keeps running sums over its samples, one
 // wavefront reduction and one LDS deposit per wavefront, one global atomic per
 // block and element.
+template <int kUnroll>
 __global__ void __launch_bounds__(kBlock) linreg_wave_kernel(LinregArgs a) {
     using Acc = BlockAccumulator<double, kWidth, Strategy::WaveThenLds, 1, 1>;
     __shared__ __attribute__((aligned(16))) double lds[kWidth];
     Acc acc(lds, 1, a.out, 1);
     const double va = a.params[0], vb = a.params[1], vc = a.params[2], vd = a.params[3];
     double sums[kWidth] = {0.0, 0.0, 0.0, 0.0, 0.0};
-    const std::size_t stride = static_cast<std::size_t>(gridDim.x) * kBlock;
-    for (std::size_t i = static_cast<std::size_t>(blockIdx.x) * kBlock + threadIdx.x; i < a.n; i += stride) {
-        const std::size_t r = row_of(a, i);
-        if (r >= a.total) continue;  // a row outside the arrays is dropped, not read
-        Variable<1, double> pa(va), pb(vb), pc(vc), pd(vd);
-        sums[4] += xad_linreg::run_loss_graph(pa, pb, pc, pd, a.x1[r], a.x2[r], a.y[r]);
-        sums[0] += pa.grad(0);
-        sums[1] += pb.grad(0);
-        sums[2] += pc.grad(0);
-        sums[3] += pd.grad(0);
+    // kUnroll samples per trip, all loads issued before the first graph runs: over a large batch the
+    // kernel is a pure read stream (24 bytes per sample) and wants that many loads in flight per
+    // lane; a small batch is latency-bound and is spread over as many lanes as possible instead
+    const std::size_t stride = static_cast<std::size_t>(gridDim.x) * kBlock * kUnroll;
+    for (std::size_t base = static_cast<std::size_t>(blockIdx.x) * kBlock * kUnroll + threadIdx.x; base < a.n; base += stride) {
+        double x1[kUnroll], x2[kUnroll], y[kUnroll];
+        bool use[kUnroll];
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            const std::size_t i = base + static_cast<std::size_t>(u) * kBlock;
+            const std::size_t r = i < a.n ? row_of(a, i) : a.total;
+            use[u] = r < a.total;  // a row outside the arrays is dropped, not read
+            x1[u] = use[u] ? __builtin_nontemporal_load(a.x1 + r) : 0.0;
+            x2[u] = use[u] ? __builtin_nontemporal_load(a.x2 + r) : 0.0;
+            y[u] = use[u] ? __builtin_nontemporal_load(a.y + r) : 0.0;
+        }
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            if (!use[u]) continue;
+            Variable<1, double> pa(va), pb(vb), pc(vc), pd(vd);
+            sums[4] += xad_linreg::run_loss_graph(pa, pb, pc, pd, x1[u], x2[u], y[u]);
+            sums[0] += pa.grad(0);
+            sums[1] += pb.grad(0);
+            sums[2] += pc.grad(0);
+            sums[3] += pd.grad(0);
+        }
     }
     acc.add(0, sums);
     acc.flush();
@@ -128,7 +145,10 @@ int launch_gradient(int strategy, const LinregArgs& a, unsigned blocks, hipStrea
             linreg_leaf_kernel<<<blocks, kBlock, 0, stream>>>(a);
             break;
         case XAD_LINREG_WAVE_LDS:
-            linreg_wave_kernel<<<blocks, kBlock, 0, stream>>>(a);
+            if (a.n >= (std::size_t(1) << 20))
+                linreg_wave_kernel<4><<<blocks, kBlock, 0, stream>>>(a);
+            else
+                linreg_wave_kernel<1><<<blocks, kBlock, 0, stream>>>(a);
             break;
         default:
             return xad::fail(XAD_ERR_INVALID_ARGUMENT, "unknown accumulation strategy %d", strategy);
