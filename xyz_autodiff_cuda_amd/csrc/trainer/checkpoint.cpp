@@ -86,6 +86,16 @@ std::string read_checkpoint(const std::string& path, CheckpointState& state) {
     if (h.num_gaussians <= 0 || h.num_gaussians > (1 << 26) || h.width <= 0 || h.height <= 0 || h.iteration < 0)
         return "checkpoint: " + path + " has a damaged header";
     const std::size_t g = static_cast<std::size_t>(h.num_gaussians);
+    {
+        // the header fixes the length of the file: check it before sizing anything by the header
+        const long at = std::ftell(f.get());
+        if (at < 0 || std::fseek(f.get(), 0, SEEK_END) != 0) return "checkpoint: cannot seek in " + path;
+        const long length = std::ftell(f.get());
+        if (std::fseek(f.get(), at, SEEK_SET) != 0) return "checkpoint: cannot seek in " + path;
+        const unsigned long long expected = sizeof(CheckpointHeader) + 4ull * 28ull * g + 4ull;
+        if (length < 0 || static_cast<unsigned long long>(length) < expected) return "checkpoint: " + path + " is truncated";
+        if (static_cast<unsigned long long>(length) > expected) return "checkpoint: " + path + " has trailing bytes";
+    }
     state.params.resize(9 * g);
     state.m.resize(9 * g);
     state.v.resize(9 * g);

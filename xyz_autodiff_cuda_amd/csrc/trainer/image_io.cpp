@@ -16,7 +16,7 @@ namespace {
 using Bytes = std::vector<unsigned char>;
 
 constexpr unsigned char kPngSignature[8] = {0x89, 'P', 'N', 'G', '\r', '\n', 0x1A, '\n'};
-constexpr std::size_t kMaxPixels = std::size_t(1) << 28;  // 16384 x 16384
+constexpr std::size_t kMaxPixels = std::size_t(1) << 26;  // 8192 x 8192
 
 std::string read_file(const std::string& path, Bytes& out) {
     std::unique_ptr<std::FILE, int (*)(std::FILE*)> f(std::fopen(path.c_str(), "rb"), &std::fclose);
