@@ -385,6 +385,37 @@ XAD_HD inline int run_case(int id, double* out) {
             put(s); put(c);
             break;
         }
+        case 15: {  // the regression network written with operators, analytic and numerical:
+                    // tests/operation/base/test_linear_regression_network.cu:39-78, parameter sets :186-196,
+                    // :211-219, :282-290, :306-314 (a, b, c, d, x1, x2, y_target)
+            const double sets[4][7] = {{1.0, 1.5, 0.5, 0.2, 2.0, 1.5, 3.0},
+                                       {0.8, 1.2, -0.3, 0.5, 1.0, 0.8, 2.5},
+                                       {10.0, 15.0, -8.0, 5.0, 20.0, -10.0, 100.0},
+                                       {0.001, 0.002, -0.001, 0.0001, 0.01, -0.01, 0.001}};
+            for (int k = 0; k < 4; ++k) {
+                for (int numerical = 0; numerical < 2; ++numerical) {
+                    double value[4] = {sets[k][0], sets[k][1], sets[k][2], sets[k][3]}, diff[4] = {0.0, 0.0, 0.0, 0.0};
+                    VariableRef<1, double> a_var(&value[0], &diff[0]), b_var(&value[1], &diff[1]), c_var(&value[2], &diff[2]),
+                        d_var(&value[3], &diff[3]);
+                    auto x1_minus_a = a_var - sets[k][4];
+                    auto x1_term = op::squared(x1_minus_a);
+                    auto x2_minus_c = c_var - sets[k][5];
+                    auto x2_squared = op::squared(x2_minus_c);
+                    auto x2_term = b_var * x2_squared;
+                    auto combined_terms = x1_term + x2_term;
+                    auto y_pred = combined_terms + d_var;
+                    auto y_diff = y_pred - sets[k][6];
+                    auto loss = op::squared(y_diff);
+                    if (numerical)
+                        loss.run_numerical(k == 3 ? 1e-8 : (k == 2 ? 1e-5 : 1e-6));
+                    else
+                        loss.run();
+                    if (!numerical) put(loss[0]);
+                    for (int j = 0; j < 4; ++j) put(diff[j]);
+                }
+            }
+            break;
+        }
         default:
             return -1;
     }
