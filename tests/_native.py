@@ -21,6 +21,9 @@ LOGICS = {
     "matvec_2x3": (24, (6, 3), 0, 2), "vecmat_3x2": (25, (3, 6), 0, 2), "generate_covariance_matrix": (26, (2, 1), 0, 4),
     "matrix_to_covariance_3param": (27, (4,), 0, 3), "scale_rotation_to_covariance_3param": (28, (2, 1), 0, 3),
     "mahalanobis_distance": (29, (2, 3), 0, 1), "mahalanobis_distance_with_center": (30, (2, 3), 2, 1),
+    # "<logic>@<size>": the same logic at another operand size
+    "exp@1": (31, (1,), 0, 1), "exp@20": (32, (20,), 0, 20), "sigmoid@1": (33, (1,), 0, 1), "sigmoid@20": (34, (20,), 0, 20),
+    "mul@1": (35, (1, 1), 0, 1), "mul@5": (36, (5, 5), 0, 5), "add@5": (37, (5, 5), 0, 5),
 }
 
 

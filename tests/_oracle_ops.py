@@ -11,6 +11,7 @@ def _arr(x, dtype):
 
 
 def evaluate(oracle, name, operands, constants=(), upstream=None, dtype=np.float64):
+    name = name.split("@")[0]  # "<logic>@<size>" is the same logic at another operand size
     dt = np.dtype(dtype)
     ops = [_arr(o, dt) for o in operands]
     k = _arr(constants, dt)
@@ -108,6 +109,7 @@ def sample_inputs(name, rng):
     from tests._native import LOGICS
 
     _, sizes, n_const, _ = LOGICS[name]
+    name = name.split("@")[0]
     lo, hi = -2.0, 2.0
     operands = [rng.uniform(lo, hi, s) for s in sizes]
     constants = rng.uniform(0.5, 2.0, n_const) * rng.choice([-1.0, 1.0], n_const) if n_const else np.zeros(0)

@@ -99,6 +99,14 @@ XAD_HD int eval_logic(int logic, const double* in, const double* up, double delt
         case 30:
             return eval_binary<T, op::MahalanobisDistanceWithCenterLogic<V2, V3>, 2, 3, 1>(
                 op::MahalanobisDistanceWithCenterLogic<V2, V3>(static_cast<T>(in[5]), static_cast<T>(in[6])), in, up, delta, out);
+        // other operand sizes of the element-wise logics: tests/operation/base/test_gradient_verification.cu:14-39, :77-86
+        case 31: return eval_unary<T, op::ExpLogic<1>, 1, 1>({}, in, up, delta, out);
+        case 32: return eval_unary<T, op::ExpLogic<20>, 20, 20>({}, in, up, delta, out);
+        case 33: return eval_unary<T, op::SigmoidLogic<1>, 1, 1>({}, in, up, delta, out);
+        case 34: return eval_unary<T, op::SigmoidLogic<20>, 20, 20>({}, in, up, delta, out);
+        case 35: return eval_binary<T, op::MulLogic<V1, V1>, 1, 1, 1>({}, in, up, delta, out);
+        case 36: return eval_binary<T, op::MulLogic<Variable<5, T>, Variable<5, T>>, 5, 5, 5>({}, in, up, delta, out);
+        case 37: return eval_binary<T, op::AddLogic<Variable<5, T>, Variable<5, T>>, 5, 5, 5>({}, in, up, delta, out);
         default: return -1;
     }
 }
