@@ -376,9 +376,11 @@ __device__ __forceinline__ float reduce_scatter9(const float (&v)[9], int lane) 
 // (the Mahalanobis backward rule, d centre = -g_q (2a dx + 2b dy, 2b dx + 2c dy),
 // d inv = g_q (dx^2, 2 dx dy, dy^2), is linear in those sums, so it is applied
 // once per Gaussian instead of once per pixel).  The nine values are reduced
-// over the wavefront by reduce_scatter9 and parked in LDS; after each chunk of
-// 64 Gaussians lane j finishes Gaussian j and adds its nine record gradients to
-// the global accumulator: one global atomic per (tile, Gaussian, field).
+// over the wavefront by reduce_scatter9 and parked in LDS; after every kPark
+// list entries lane j finishes entry j of the group, and the group's record
+// gradients are added to the global accumulator with consecutive lanes on
+// consecutive fields of consecutive entries: one atomic per (tile, Gaussian,
+// field), about seven accumulator rows (cache lines) per instruction.
 __global__ void __launch_bounds__(kChunk) render_backward_kernel(
     int width, int height, int tiles_x, int tiles, const std::uint32_t* __restrict__ range_begin,
     const std::uint32_t* __restrict__ range_end, const std::uint32_t* __restrict__ sorted_ids,
@@ -447,85 +449,85 @@ __global__ void __launch_bounds__(kChunk) render_backward_kernel(
 
         // groups of up to kPark entries, back to front; all but the last-staged one are full
         for (int group_end = count; group_end > 0;) {
-        const int group_first = (group_end - 1) / kPark * kPark;
-        for (int j = group_end - 1; j >= group_first; --j) {
-            const std::uint32_t position = chunk_first + j;
-            const Staged r = staged[j];
-            // exponent of the falloff as a polynomial in dx: (a_s dx + e) dx + f
-            const float dy = py - r.cy;
-            const float e = r.b2_s * dy;
-            const float f = r.c_s * dy * dy;
-            const float dx0 = px0 - r.cx;
-            float through[kLanePixels];  // d loss / d alpha0 of this Gaussian, per pixel
-            float colour[3] = {0.f, 0.f, 0.f};
+            const int group_first = (group_end - 1) / kPark * kPark;
+            for (int j = group_end - 1; j >= group_first; --j) {
+                const std::uint32_t position = chunk_first + j;
+                const Staged r = staged[j];
+                // exponent of the falloff as a polynomial in dx: (a_s dx + e) dx + f
+                const float dy = py - r.cy;
+                const float e = r.b2_s * dy;
+                const float f = r.c_s * dy * dy;
+                const float dx0 = px0 - r.cx;
+                float through[kLanePixels];  // d loss / d alpha0 of this Gaussian, per pixel
+                float colour[3] = {0.f, 0.f, 0.f};
 #pragma unroll
-            for (int p = 0; p < kLanePixels; ++p) {
-                // A pixel is idle until the walk reaches the last Gaussian it composited, and
-                // active from there on.  While idle, alpha = 0 leaves T and D at their initial
-                // values, so no branch is needed.
-                const bool active = position < used[p];
-                const float dx = dx0 + static_cast<float>(p);
-                const float falloff = math::fp32::exp2_raw(::fmaf(::fmaf(r.a_s, dx, e), dx, f));
-                const float a = falloff * r.alpha0;
-                const bool clamped = a > kAlphaMax;
-                const float alpha = active ? __builtin_fminf(a, kAlphaMax) : 0.f;
-                const float inv = __builtin_amdgcn_rcpf(1.f - alpha);
-                const float T_front = T[p] * inv;  // transmittance in front of this Gaussian
-                const float dot = ::fmaf(dC[p][2], r.blue, ::fmaf(dC[p][1], r.green, dC[p][0] * r.red));
-                // d loss / d alpha = T_front (dC . colour) - (dC . colour behind) / (1 - alpha)
-                //                  = T_front dot + D inv
-                const float d_alpha = ::fmaf(D[p], inv, T_front * dot);
-                const float weight = alpha * T_front;
-                D[p] = ::fmaf(-weight, dot, D[p]);
-                T[p] = T_front;
+                for (int p = 0; p < kLanePixels; ++p) {
+                    // A pixel is idle until the walk reaches the last Gaussian it composited, and
+                    // active from there on.  While idle, alpha = 0 leaves T and D at their initial
+                    // values, so no branch is needed.
+                    const bool active = position < used[p];
+                    const float dx = dx0 + static_cast<float>(p);
+                    const float falloff = math::fp32::exp2_raw(::fmaf(::fmaf(r.a_s, dx, e), dx, f));
+                    const float a = falloff * r.alpha0;
+                    const bool clamped = a > kAlphaMax;
+                    const float alpha = active ? __builtin_fminf(a, kAlphaMax) : 0.f;
+                    const float inv = __builtin_amdgcn_rcpf(1.f - alpha);
+                    const float T_front = T[p] * inv;  // transmittance in front of this Gaussian
+                    const float dot = ::fmaf(dC[p][2], r.blue, ::fmaf(dC[p][1], r.green, dC[p][0] * r.red));
+                    // d loss / d alpha = T_front (dC . colour) - (dC . colour behind) / (1 - alpha)
+                    //                  = T_front dot + D inv
+                    const float d_alpha = ::fmaf(D[p], inv, T_front * dot);
+                    const float weight = alpha * T_front;
+                    D[p] = ::fmaf(-weight, dot, D[p]);
+                    T[p] = T_front;
 #pragma unroll
-                for (int c = 0; c < 3; ++c) colour[c] = ::fmaf(weight, dC[p][c], colour[c]);
-                through[p] = (active && !clamped) ? d_alpha * falloff : 0.f;
+                    for (int c = 0; c < 3; ++c) colour[c] = ::fmaf(weight, dC[p][c], colour[c]);
+                    through[p] = (active && !clamped) ? d_alpha * falloff : 0.f;
+                }
+                // Moments of `through` over the lane's four pixels (offsets 0..3 from dx0) give the five
+                // sums  sum t dx^i dy^j  the Mahalanobis backward rule needs; their common factor
+                // d alpha / d q / falloff = -alpha0 / 2 is applied once per Gaussian below.
+                const float m0 = (through[0] + through[1]) + (through[2] + through[3]);
+                const float m1 = ::fmaf(3.f, through[3], ::fmaf(2.f, through[2], through[1]));
+                const float m2 = ::fmaf(9.f, through[3], ::fmaf(4.f, through[2], through[1]));
+                const float sx = ::fmaf(dx0, m0, m1);
+                const float sy = dy * m0;
+                const float v[9] = {sx, sy, ::fmaf(dx0, sx + m1, m2), dy * sx, dy * sy, colour[0], colour[1], colour[2], m0};
+                const float mine = reduce_scatter9(v, lane);
+                if ((lane & 15) < 9) parked[j - group_first][lane >> 4][lane & 15] = mine;
             }
-            // Moments of `through` over the lane's four pixels (offsets 0..3 from dx0) give the five
-            // sums  sum t dx^i dy^j  the Mahalanobis backward rule needs; their common factor
-            // d alpha / d q / falloff = -alpha0 / 2 is applied once per Gaussian below.
-            const float m0 = (through[0] + through[1]) + (through[2] + through[3]);
-            const float m1 = ::fmaf(3.f, through[3], ::fmaf(2.f, through[2], through[1]));
-            const float m2 = ::fmaf(9.f, through[3], ::fmaf(4.f, through[2], through[1]));
-            const float sx = ::fmaf(dx0, m0, m1);
-            const float sy = dy * m0;
-            const float v[9] = {sx, sy, ::fmaf(dx0, sx + m1, m2), dy * sx, dy * sy, colour[0], colour[1], colour[2], m0};
-            const float mine = reduce_scatter9(v, lane);
-            if ((lane & 15) < 9) parked[j - group_first][lane >> 4][lane & 15] = mine;
-        }
-        const int members = group_end - group_first;
-        __syncthreads();
-        if (lane < members) {
-            float s[9];
+            const int members = group_end - group_first;
+            __syncthreads();
+            if (lane < members) {
+                float s[9];
 #pragma unroll
-            for (int k = 0; k < 9; ++k) s[k] = (parked[lane][0][k] + parked[lane][1][k]) + (parked[lane][2][k] + parked[lane][3][k]);
-            const Staged r = staged[group_first + lane];
-            const float g_q_scale = -0.5f * r.alpha0;
+                for (int k = 0; k < 9; ++k) s[k] = (parked[lane][0][k] + parked[lane][1][k]) + (parked[lane][2][k] + parked[lane][3][k]);
+                const Staged r = staged[group_first + lane];
+                const float g_q_scale = -0.5f * r.alpha0;
 #pragma unroll
-            for (int k = 0; k < 5; ++k) s[k] *= g_q_scale;
-            const float out[kRecordGrads] = {
-                -(2.f * r.a * s[0] + 2.f * r.b * s[1]),  // d centre x
-                -(2.f * r.b * s[0] + 2.f * r.c * s[1]),  // d centre y
-                s[2], 2.f * s[3], s[4],                  // d inverse covariance
-                s[5], s[6], s[7],                        // d colour
-                s[8],                                    // d alpha0
-            };
+                for (int k = 0; k < 5; ++k) s[k] *= g_q_scale;
+                const float out[kRecordGrads] = {
+                    -(2.f * r.a * s[0] + 2.f * r.b * s[1]),  // d centre x
+                    -(2.f * r.b * s[0] + 2.f * r.c * s[1]),  // d centre y
+                    s[2], 2.f * s[3], s[4],                  // d inverse covariance
+                    s[5], s[6], s[7],                        // d colour
+                    s[8],                                    // d alpha0
+                };
 #pragma unroll
-            for (int k = 0; k < kRecordGrads; ++k) parked[lane][0][k] = out[k];
-        }
-        __syncthreads();
-        // The lanes of one atomic instruction take consecutive fields of consecutive list entries, so
-        // an instruction touches about seven accumulator rows (cache lines) instead of 64.
-        for (int item = lane; item < members * kRecordGrads; item += kChunk) {
-            const int entry = item / kRecordGrads, field = item - entry * kRecordGrads;
-            const float value = parked[entry][0][field];
-            if (value != 0.f)
-                detail::atomic_add(
-                    record_grads + static_cast<std::size_t>(staged_id[group_first + entry]) * kRecordGradStride + field, value);
-        }
-        __syncthreads();  // the next group parks into the same rows
-        group_end = group_first;
+                for (int k = 0; k < kRecordGrads; ++k) parked[lane][0][k] = out[k];
+            }
+            __syncthreads();
+            // The lanes of one atomic instruction take consecutive fields of consecutive list entries, so
+            // an instruction touches about seven accumulator rows (cache lines) instead of 64.
+            for (int item = lane; item < members * kRecordGrads; item += kChunk) {
+                const int entry = item / kRecordGrads, field = item - entry * kRecordGrads;
+                const float value = parked[entry][0][field];
+                if (value != 0.f)
+                    detail::atomic_add(
+                        record_grads + static_cast<std::size_t>(staged_id[group_first + entry]) * kRecordGradStride + field, value);
+            }
+            __syncthreads();  // the next group parks into the same rows
+            group_end = group_first;
         }
     }
 }
