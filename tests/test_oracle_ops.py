@@ -20,6 +20,7 @@ NAMES = sorted(_native.LOGICS)
 
 
 def _numpy_forward(name, ops, k):
+    name = name.split("@")[0]  # "<logic>@<size>": the same logic at another operand size
     a = ops[0]
     b = ops[1] if len(ops) > 1 else None
     if name == "exp": return np.exp(a)
