@@ -365,6 +365,20 @@ def main():
         torch.cuda.synchronize()
         alt["problems_per_lane=%d" % lanes] = algorithmic_bytes / (a.elapsed_time(b) / 10 / 1e3) / 1e9
 
+    # the store policy of the default kernel, measured again: alternating rounds of ten launches each
+    policy_ms = {name: [] for name in chain.STORE_POLICIES}
+    for _ in range(3):
+        for name in chain.STORE_POLICIES:
+            chain.store_policy_probe(ins, outs, name)
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            for _ in range(10):
+                chain.store_policy_probe(ins, outs, name)
+            b.record()
+            torch.cuda.synchronize()
+            policy_ms[name].append(a.elapsed_time(b) / 10)
+    store_policy = {name: algorithmic_bytes / (sorted(v)[1] / 1e3) / 1e9 for name, v in policy_ms.items()}
+
     record = {
         "metric": "per-thread fwd+bwd evals/sec",
         "value": n * args.steps / wall,
@@ -396,6 +410,7 @@ def main():
         },
         "outputs_finite": finite,
         "mapping_GBps": alt,
+        "store_policy_GBps": store_policy,
     }
     record["accumulate"] = accumulate_report(ins, args.seed, with_oracle=not args.no_cpu)
     if not args.no_cpu:

@@ -353,6 +353,19 @@ int xad_host_linreg_gradient_f64(size_t n, size_t total,
  */
 int xad_probe_lds_atomic_cycles(int element, int pattern, double* cycles_per_instruction);
 
+/* Hardware probe behind the default kernel of xad_chain_forward_backward_f32: the
+ * same kernel (one problem per lane, non-temporal loads) with its seven results
+ * stored as 0 write-through stores (relaxed atomic stores at agent scope, the
+ * library's choice), 1 plain stores, 2 non-temporal stores.  Same arguments and
+ * results as xad_chain_forward_backward_f32; only the time differs.  No
+ * counterpart in the reference.
+ */
+int xad_probe_chain_store_policy(int policy, size_t n,
+                                 const float* sx, const float* sy, const float* theta,
+                                 const float* o, const float* px, const float* py,
+                                 float* w, float* d_sx, float* d_sy, float* d_theta,
+                                 float* d_o, float* d_px, float* d_py, void* stream);
+
 /* ---------------------------------------------------------------------------
  * Synthetic inputs: counter-based generator, element i of a fill is a pure
  * function of (seed, stream_id, i).  The reference seeds std::mt19937 on the

@@ -71,6 +71,23 @@ def test_both_lane_mappings_and_unaligned_buffers_agree_bitwise(gpu, oracle):
     assert np.array_equal(a, c)
 
 
+def test_store_policies_of_the_probe_agree_bitwise(gpu, xad):
+    """xad_probe_chain_store_policy changes how results are stored, never what is stored."""
+    import torch
+
+    from xyz_autodiff_cuda_amd import chain
+
+    n = 70_001
+    ins = [torch.from_numpy(a).to(gpu) for a in chain_inputs(n, seed=12)]
+    want = torch.stack(chain.forward_backward(ins))
+    for policy in chain.STORE_POLICIES:
+        outs = [torch.full((n,), float("nan"), dtype=torch.float32, device=gpu) for _ in range(7)]
+        chain.store_policy_probe(ins, outs, policy)
+        assert torch.equal(torch.stack(outs), want), policy
+    with pytest.raises(xad.XadError, match="policy"):
+        chain.store_policy_probe(ins, outs, 7)
+
+
 def test_device_matches_host_build_of_the_same_templates(gpu, xad):
     from xyz_autodiff_cuda_amd import chain
 

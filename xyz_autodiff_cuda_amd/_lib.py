@@ -66,6 +66,7 @@ SIGNATURES = {
     "xad_linreg_gradient_f64": [_int, _sz, _sz, _vp, _vp, _vp, _vp, _vp, _vp, _vp],
     "xad_linreg_sgd_f64": [_sz, _vp, _vp, _vp, _vp, _int, _int, ctypes.c_double, ctypes.c_double, _u64, _vp, _vp],
     "xad_host_linreg_gradient_f64": [_sz, _sz, _vp, _vp, _vp, _vp, _vp, _vp],
+    "xad_probe_chain_store_policy": [_int, _sz] + [_vp] * 13 + [_vp],
     "xad_probe_lds_atomic_cycles": [_int, _int, ctypes.POINTER(ctypes.c_double)],
     "xad_rng_zipf_i32": [_vp, _sz, _u64, _u64, _int, ctypes.c_double, _vp],
     "xad_rng_uniform_f32": [_vp, _sz, _u64, _u64, _flt, _flt, _vp],

@@ -58,6 +58,26 @@ def forward_backward(inputs, outputs=None, stream=None, problems_per_lane=None):
     return outputs
 
 
+STORE_POLICIES = {"write_through": 0, "plain": 1, "non_temporal": 2}
+
+
+def store_policy_probe(inputs, outputs, policy, stream=None):
+    """The default kernel with another store policy (see xad_probe_chain_store_policy); same results."""
+    import torch
+
+    lib = _lib.load()
+    n = inputs[0].numel()
+    for t, name in zip(list(inputs) + list(outputs), INPUT_NAMES + OUTPUT_NAMES):
+        _require_cuda_f32(t, name, n)
+    s = stream if stream is not None else torch.cuda.current_stream(inputs[0].device)
+    ptrs = [t.data_ptr() for t in inputs] + [t.data_ptr() for t in outputs]
+    with torch.cuda.device(inputs[0].device):
+        status = lib.xad_probe_chain_store_policy(STORE_POLICIES[policy] if isinstance(policy, str) else int(policy), n, *ptrs,
+                                                  s.cuda_stream)
+    _lib.check(status, "xad_probe_chain_store_policy")
+    return outputs
+
+
 def host_forward_backward(inputs, dtype=np.float32, num_threads=0):
     """The same templates compiled for the host cores; numpy in, numpy out."""
     lib = _lib.load()

@@ -68,7 +68,22 @@ __global__ void __launch_bounds__(kQuadBlock) chain_quad_kernel(ChainBuffers buf
     for (int a = 0; a < 7; ++a) store4_stream(buf.out[a], g, out[a]);
 }
 
-// One lane, one problem, 4-byte accesses; problems first .. n-1.  Non-temporal loads, write-through stores.
+// How the seven results are stored.  WriteThrough is what the library uses; the other two exist
+// so that the choice can be measured again (xad_probe_chain_store_policy).
+enum class StorePolicy { WriteThrough = 0, Plain = 1, NonTemporal = 2 };
+
+template <StorePolicy P>
+__device__ __forceinline__ void store_result(float* address, float value) {
+    if constexpr (P == StorePolicy::WriteThrough)
+        __hip_atomic_store(address, value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // global_store_dword ... sc1
+    else if constexpr (P == StorePolicy::Plain)
+        *address = value;
+    else
+        __builtin_nontemporal_store(value, address);
+}
+
+// One lane, one problem, 4-byte accesses; problems first .. n-1.  Non-temporal loads.
+template <StorePolicy P>
 __global__ void __launch_bounds__(kSingleBlock) chain_single_kernel(ChainBuffers buf, std::size_t first, std::size_t n) {
     const std::size_t i = first + static_cast<std::size_t>(blockIdx.x) * kSingleBlock + threadIdx.x;
     if (i >= n) return;
@@ -78,7 +93,7 @@ __global__ void __launch_bounds__(kSingleBlock) chain_single_kernel(ChainBuffers
     const auto r = xad_chain::forward_backward<float>(x[0], x[1], x[2], x[3], x[4], x[5]);
     const float y[7] = {r.w, r.d_sx, r.d_sy, r.d_theta, r.d_o, r.d_px, r.d_py};
 #pragma unroll
-    for (int a = 0; a < 7; ++a) __hip_atomic_store(buf.out[a] + i, y[a], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    for (int a = 0; a < 7; ++a) store_result<P>(buf.out[a] + i, y[a]);
 }
 
 // Plain copy with the chain kernel's access pattern (4 bytes per lane, non-temporal):
@@ -153,14 +168,36 @@ int launch_chain(std::size_t n, const ChainBuffers& buf, int problems_per_lane, 
     }
     const std::size_t done = groups * 4;
     if (done < n) {
-        hipLaunchKernelGGL(chain_single_kernel, dim3(xad::blocks_for(n - done, kSingleBlock)), dim3(kSingleBlock), 0,
-                           s, buf, done, n);
+        hipLaunchKernelGGL(chain_single_kernel<StorePolicy::WriteThrough>, dim3(xad::blocks_for(n - done, kSingleBlock)),
+                           dim3(kSingleBlock), 0, s, buf, done, n);
         XAD_HIP_TRY(hipGetLastError());
     }
     return XAD_OK;
 }
 
 }  // namespace
+
+extern "C" int xad_probe_chain_store_policy(int policy, std::size_t n, const float* sx, const float* sy,
+                                            const float* theta, const float* o, const float* px, const float* py,
+                                            float* w, float* d_sx, float* d_sy, float* d_theta, float* d_o,
+                                            float* d_px, float* d_py, void* stream) {
+    const char* who = "xad_probe_chain_store_policy";
+    const ChainBuffers buf{{sx, sy, theta, o, px, py}, {w, d_sx, d_sy, d_theta, d_o, d_px, d_py}};
+    if (n == 0) return XAD_OK;
+    for (int a = 0; a < 6; ++a) XAD_REQUIRE(buf.in[a], "%s: input array %d is null", who, a);
+    for (int a = 0; a < 7; ++a) XAD_REQUIRE(buf.out[a], "%s: output array %d is null", who, a);
+    XAD_REQUIRE(n <= 0x7fffffffull * 64, "%s: n = %zu exceeds the grid limit", who, n);
+    const dim3 grid(xad::blocks_for(n, kSingleBlock)), block(kSingleBlock);
+    hipStream_t s = xad::as_stream(stream);
+    switch (policy) {
+        case 0: hipLaunchKernelGGL(chain_single_kernel<StorePolicy::WriteThrough>, grid, block, 0, s, buf, 0, n); break;
+        case 1: hipLaunchKernelGGL(chain_single_kernel<StorePolicy::Plain>, grid, block, 0, s, buf, 0, n); break;
+        case 2: hipLaunchKernelGGL(chain_single_kernel<StorePolicy::NonTemporal>, grid, block, 0, s, buf, 0, n); break;
+        default: return xad::fail(XAD_ERR_INVALID_ARGUMENT, "%s: policy must be 0, 1 or 2, got %d", who, policy);
+    }
+    XAD_HIP_TRY(hipGetLastError());
+    return XAD_OK;
+}
 
 extern "C" int xad_chain_forward_backward_f32(std::size_t n, const float* sx, const float* sy, const float* theta,
                                               const float* o, const float* px, const float* py, float* w,
