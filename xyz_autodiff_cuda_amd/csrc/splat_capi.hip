@@ -111,10 +111,9 @@ int bin(xad_splat_context* c, const float* params, const float* depth, hipStream
     const bool had_order = c->order_valid;
     if (!had_order)
         if (int st = order_by_depth(c, depth, s)) return st;
-    std::uint32_t* depth_changed = c->offsets + c->G + 1;
-    XAD_HIP_TRY(hipMemsetAsync(depth_changed, 0, sizeof(std::uint32_t), s));
+    std::uint32_t* depth_changed = c->offsets + c->G + 1;  // zero at creation, reset by every emit
     if (int st = launch_project(s, c->G, params, depth, c->ordered_depth, depth_changed, c->width, c->height, c->records,
-                                c->rects, c->counts))
+                                c->rects, c->counts, c->record_grads, c->loss))
         return st;
     mark(c, 1, s);
     // The order of the previous call is used on the assumption that the depths are the same; the
@@ -130,14 +129,13 @@ int bin(xad_splat_context* c, const float* params, const float* depth, hipStream
         if (int st = allocate_pair_buffers(c, static_cast<std::uint32_t>(want))) return st;
     }
     if (int st = launch_emit(s, c->G, c->by_depth, c->rects, c->offsets, c->tiles_x, c->wide_keys, c->keys, c->ids,
-                             c->capacity))
+                             c->capacity, c->range_begin, c->tiles * 2, depth_changed))
         return st;
     mark(c, 2, s);
     if (int st = sort_pairs(s, c->sort_temp, c->sort_bytes, c->wide_keys, c->keys, c->keys_sorted, c->ids, c->ids_sorted,
                             c->pairs, c->key_bits))
         return st;
     mark(c, 3, s);
-    XAD_HIP_TRY(hipMemsetAsync(c->range_begin, 0, sizeof(std::uint32_t) * c->tiles * 2, s));
     if (int st = launch_ranges(s, c->pairs, c->wide_keys, c->keys_sorted, c->range_begin, c->range_end)) return st;
     mark(c, 4, s);
     return XAD_OK;
@@ -214,6 +212,8 @@ extern "C" int xad_splat_create(int width, int height, int num_gaussians, std::s
         st = xad::fail(XAD_ERR_HIP, "%s: hipMemset failed", who);
     if (st == XAD_OK && hipMemset(c->counts_by_depth, 0, sizeof(std::uint32_t) * (G + 1)) != hipSuccess)
         st = xad::fail(XAD_ERR_HIP, "%s: hipMemset failed", who);
+    if (st == XAD_OK && hipMemset(c->offsets, 0, sizeof(std::uint32_t) * (G + 2)) != hipSuccess)  // includes the flag
+        st = xad::fail(XAD_ERR_HIP, "%s: hipMemset failed", who);
     if (st == XAD_OK) {
         const std::size_t hint = pair_capacity_hint ? pair_capacity_hint : G * 8 + 1024;
         st = allocate_pair_buffers(c, static_cast<std::uint32_t>(hint < 0xfffffff0ull ? hint : 0xfffffff0ull));
@@ -285,8 +285,6 @@ extern "C" int xad_splat_step(xad_splat_context* c, const float* params, const f
                                        image, c->final_T, c->n_contrib))
         return st;
     mark(c, 5, s);
-    XAD_HIP_TRY(hipMemsetAsync(c->record_grads, 0, sizeof(float) * static_cast<std::size_t>(c->G) * kRecordGradStride, s));
-    XAD_HIP_TRY(hipMemsetAsync(c->loss, 0, sizeof(double), s));
     if (int st = launch_render_backward(s, c->width, c->height, c->range_begin, c->range_end, c->ids_sorted, c->records,
                                         image, target, c->final_T, c->n_contrib, c->record_grads, c->loss))
         return st;

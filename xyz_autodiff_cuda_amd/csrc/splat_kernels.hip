@@ -33,9 +33,17 @@ __global__ void __launch_bounds__(256) project_kernel(int G, const float* __rest
                                                       const float* __restrict__ ordered_depth,
                                                       std::uint32_t* __restrict__ depth_changed, int width, int height,
                                                       Record* __restrict__ records, TileRect* __restrict__ rects,
-                                                      std::uint32_t* __restrict__ counts) {
+                                                      std::uint32_t* __restrict__ counts,
+                                                      float* __restrict__ record_grads, double* __restrict__ loss) {
     const int g = blockIdx.x * 256 + threadIdx.x;
     if (g >= G) return;
+    // what the compositing backward adds into starts from zero: this Gaussian's accumulator row, the loss
+    {
+        float4* row = reinterpret_cast<float4*>(record_grads + static_cast<std::size_t>(g) * kRecordGradStride);
+#pragma unroll
+        for (int k = 0; k < kRecordGradStride / 4; ++k) row[k] = float4{0.f, 0.f, 0.f, 0.f};
+        if (g == 0) *loss = 0.0;
+    }
     // the depth order of the previous call stays valid while every depth keeps its bits
     if (__builtin_bit_cast(std::uint32_t, depth[g]) != __builtin_bit_cast(std::uint32_t, ordered_depth[g]))
         atomicOr(depth_changed, 1u);
@@ -129,9 +137,14 @@ __global__ void __launch_bounds__(256) emit_kernel(int G, const std::uint32_t* _
                                                    const TileRect* __restrict__ rects,
                                                    const std::uint32_t* __restrict__ offsets, int tiles_x,
                                                    Key* __restrict__ keys, std::uint32_t* __restrict__ values,
-                                                   std::uint32_t capacity) {
+                                                   std::uint32_t capacity, std::uint32_t* __restrict__ tile_ranges,
+                                                   int range_words, std::uint32_t* __restrict__ depth_changed) {
     const int i = blockIdx.x * 256 + threadIdx.x;
     const int lane = threadIdx.x & 63;
+    // housekeeping for what runs later in the step: empty tile ranges (tiles without pairs keep
+    // them), and the depth-changed flag, which the host has read by now, back to zero
+    for (int t = i; t < range_words; t += static_cast<int>(gridDim.x) * 256) tile_ranges[t] = 0;
+    if (i == 0) *depth_changed = 0;
     std::uint32_t g = 0, at = 0, count = 0;
     int x0 = 0, y0 = 0, columns = 1;
     if (i < G) {
@@ -581,9 +594,9 @@ __global__ void __launch_bounds__(256) gaussian_backward_kernel(int G, const flo
 
 int launch_project(hipStream_t s, int G, const float* params, const float* depth, const float* ordered_depth,
                    std::uint32_t* depth_changed, int width, int height, Record* records, TileRect* rects,
-                   std::uint32_t* counts) {
+                   std::uint32_t* counts, float* record_grads, double* loss) {
     hipLaunchKernelGGL(project_kernel, dim3(xad::blocks_for(G, 256)), dim3(256), 0, s, G, params, depth, ordered_depth,
-                       depth_changed, width, height, records, rects, counts);
+                       depth_changed, width, height, records, rects, counts, record_grads, loss);
     XAD_HIP_TRY(hipGetLastError());
     return XAD_OK;
 }
@@ -603,13 +616,16 @@ int launch_permute_counts(hipStream_t s, int G, const std::uint32_t* by_depth, c
 }
 
 int launch_emit(hipStream_t s, int G, const std::uint32_t* by_depth, const TileRect* rects, const std::uint32_t* offsets,
-                int tiles_x, bool wide_keys, void* keys, std::uint32_t* values, std::uint32_t capacity) {
+                int tiles_x, bool wide_keys, void* keys, std::uint32_t* values, std::uint32_t capacity,
+                std::uint32_t* tile_ranges, int range_words, std::uint32_t* depth_changed) {
     if (wide_keys)
         hipLaunchKernelGGL(emit_kernel<std::uint32_t>, dim3(xad::blocks_for(G, 256)), dim3(256), 0, s, G, by_depth, rects,
-                           offsets, tiles_x, static_cast<std::uint32_t*>(keys), values, capacity);
+                           offsets, tiles_x, static_cast<std::uint32_t*>(keys), values, capacity, tile_ranges, range_words,
+                           depth_changed);
     else
         hipLaunchKernelGGL(emit_kernel<std::uint16_t>, dim3(xad::blocks_for(G, 256)), dim3(256), 0, s, G, by_depth, rects,
-                           offsets, tiles_x, static_cast<std::uint16_t*>(keys), values, capacity);
+                           offsets, tiles_x, static_cast<std::uint16_t*>(keys), values, capacity, tile_ranges, range_words,
+                           depth_changed);
     XAD_HIP_TRY(hipGetLastError());
     return XAD_OK;
 }

@@ -11,10 +11,11 @@
 
 namespace xad_splat {
 
-// Also sets *depth_changed to 1 if any depth differs (bitwise) from ordered_depth.
+// Also sets *depth_changed to 1 if any depth differs (bitwise) from ordered_depth, and zeroes
+// record_grads (G rows of kRecordGradStride floats) and *loss for the compositing backward.
 int launch_project(hipStream_t s, int G, const float* params, const float* depth, const float* ordered_depth,
                    std::uint32_t* depth_changed, int width, int height, Record* records, TileRect* rects,
-                   std::uint32_t* counts);
+                   std::uint32_t* counts, float* record_grads, double* loss);
 // Depth order: keys[g] = order-preserving bits of depth[g], identity[g] = g; the stable sort of
 // those pairs gives by_depth.  counts_by_depth[i] = counts[by_depth[i]].
 int launch_depth_keys(hipStream_t s, int G, const float* depth, std::uint32_t* keys, std::uint32_t* identity);
@@ -22,8 +23,10 @@ int launch_permute_counts(hipStream_t s, int G, const std::uint32_t* by_depth, c
                           std::uint32_t* counts_by_depth);
 // Pairs are emitted in depth order with the tile index as key: 16 bits wide, or 32 (wide_keys)
 // when there are more than 65 536 tiles.
+// Also zeroes the range_words words of tile_ranges and resets *depth_changed.
 int launch_emit(hipStream_t s, int G, const std::uint32_t* by_depth, const TileRect* rects, const std::uint32_t* offsets,
-                int tiles_x, bool wide_keys, void* keys, std::uint32_t* values, std::uint32_t capacity);
+                int tiles_x, bool wide_keys, void* keys, std::uint32_t* values, std::uint32_t capacity,
+                std::uint32_t* tile_ranges, int range_words, std::uint32_t* depth_changed);
 int launch_ranges(hipStream_t s, std::uint32_t K, bool wide_keys, const void* keys, std::uint32_t* range_begin,
                   std::uint32_t* range_end);
 int launch_render_forward(hipStream_t s, int width, int height, const std::uint32_t* range_begin,
