@@ -17,7 +17,11 @@
  *     (The reference's host helpers throw std::runtime_error instead,
  *     include/xyz_autodiff/util/error_checker.cuh:9-20.)
  *   - nothing here falls back to the CPU: an entry point without the xad_host_
- *     prefix either runs on the GPU or fails.
+ *     prefix either runs on the GPU or fails;
+ *   - the library keeps no global state besides the thread-local error text:
+ *     calls from several host threads are independent as long as they do not
+ *     share a context object (xad_splat_context, xad_trainer), which serves one
+ *     call at a time, or write to the same device memory.
  */
 #ifndef XAD_CAPI_H
 #define XAD_CAPI_H
