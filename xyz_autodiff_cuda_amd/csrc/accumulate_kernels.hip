@@ -67,17 +67,31 @@ __global__ void __launch_bounds__(kBlock) accumulate_kernel(AccumulateArgs a) {
 
     const std::size_t begin = static_cast<std::size_t>(blockIdx.x >> a.part_shift) * a.per_block;
     const std::size_t end = begin + a.per_block < a.n ? begin + a.per_block : a.n;
-    for (std::size_t base = begin; base < end; base += kBlock) {
+    // The inputs of the next trip are requested before the arithmetic of this one, so that a lane has
+    // two trips' worth of loads in flight instead of waiting for memory twice per trip (slot, then inputs).
+    struct Inputs {
+        int slot;  // as stored; -1 past the end
+        float x[6];
+    };
+    auto fetch = [&](std::size_t base) {
+        Inputs in{-1, {0.f, 0.f, 0.f, 0.f, 0.f, 0.f}};
         const std::size_t i = base + threadIdx.x;
-        int slot = -1;
-        float g[kWidth] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-        // a slot outside [0, num_slots) is dropped rather than written out of bounds
-        if (i < end) slot = part.row_of(__builtin_nontemporal_load(a.slot + i), a);
-        if (slot >= 0) {
-            float x[6];
+        if (i < end) {
+            in.slot = __builtin_nontemporal_load(a.slot + i);
 #pragma unroll
-            for (int k = 0; k < 6; ++k) x[k] = __builtin_nontemporal_load(a.in[k] + i);
-            const auto r = xad_chain::forward_backward<float>(x[0], x[1], x[2], x[3], x[4], x[5]);
+            for (int k = 0; k < 6; ++k) in.x[k] = __builtin_nontemporal_load(a.in[k] + i);
+        }
+        return in;
+    };
+    Inputs current = fetch(begin);
+    for (std::size_t base = begin; base < end; base += kBlock) {
+        const Inputs next = fetch(base + kBlock);
+        // a slot outside [0, num_slots) is dropped rather than written out of bounds
+        const int slot = part.row_of(current.slot, a);
+        float g[kWidth] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        if (slot >= 0) {
+            const auto r = xad_chain::forward_backward<float>(current.x[0], current.x[1], current.x[2], current.x[3],
+                                                              current.x[4], current.x[5]);
             g[0] = r.d_sx;
             g[1] = r.d_sy;
             g[2] = r.d_theta;
@@ -86,6 +100,7 @@ __global__ void __launch_bounds__(kBlock) accumulate_kernel(AccumulateArgs a) {
             g[5] = r.d_py;
         }
         acc.add(slot, g);
+        current = next;
     }
     acc.flush();
 }
@@ -225,7 +240,7 @@ extern "C" int xad_accumulate_chain_gradients_f32(int strategy, std::size_t n, c
         lds += BlockAccumulator<float, kWidth>::spill_bytes(kBlock);
     }
     XAD_REQUIRE(lds <= kMaxLdsBytes, "%s: LDS table of %zu bytes does not fit", who, lds);
-    const int per_cu = lds <= 32 * 1024 ? 2 : 1;
+    const int per_cu = lds <= 72 * 1024 ? 2 : 1;  // two 1024-lane blocks fill a CU; 160 KiB of LDS hold two tables up to 72 KiB
     if (a.spill_offset) {
         switch (strategy) {
             case XAD_ACCUMULATE_WAVE_LDS:
