@@ -124,8 +124,10 @@ int xad_host_chain_forward_backward_f64(size_t n,
  *                   those fit in 48 KiB so that lanes sharing a slot do not share an
  *                   address; up to 6144 slots the slots are
  *                   dealt to two fp64 tables served by two sets of blocks; beyond
- *                   that 4096 fp32 rows are claimed on first use and the rest falls
- *                   through to HBM.  LDS_F32 forces one fp32 table (up to 6144 slots);
+ *                   that rows are claimed on first use (2048 fp64 rows up to
+ *                   262 144 slots, 4096 fp32 rows above) and the rest falls
+ *                   through to HBM.  LDS_F32 forces fp32 tables (one for all slots
+ *                   up to 6144, 4096 claimed rows above);
  *   WAVE_LDS        DPP pre-reduction of equal slots inside each wavefront (groups
  *                   of >= 4 lanes, up to eight groups per call), then as LDS;
  *                   WAVE_LDS_SHALLOW: at most two groups;

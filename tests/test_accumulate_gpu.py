@@ -59,7 +59,7 @@ def _assert_close(got, ref, sum_tol):
 
 
 @pytest.mark.parametrize("strategy", STAGED)
-@pytest.mark.parametrize("num_slots", [1, 3, 64, 3072, 3073, 4096, 5001, 6144, 7000, 262144])
+@pytest.mark.parametrize("num_slots", [1, 3, 64, 3072, 3073, 4096, 5001, 6144, 7000, 262144, 600000])
 def test_staged_strategies_match_fp64_sums(gpu, oracle, strategy, num_slots):
     n = 1_000_003
     inputs = chain_inputs(n, seed=50 + num_slots % 97)
@@ -78,7 +78,7 @@ def test_naive_global_atomics(gpu, oracle, strategy, num_slots):
     _assert_close(_run(gpu, inputs, slot, num_slots, strategy), ref, 1e-2)
 
 
-@pytest.mark.parametrize("num_slots", [10, 5001])  # one table; slots dealt to two tables
+@pytest.mark.parametrize("num_slots", [10, 5001, 7000])  # one table; slots dealt to two tables; claimed rows
 def test_adds_to_existing_values_and_ignores_out_of_range_slots(gpu, oracle, num_slots):
     n = 100_000
     inputs = chain_inputs(n, seed=3)

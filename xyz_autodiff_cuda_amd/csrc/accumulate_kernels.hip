@@ -212,7 +212,7 @@ extern "C" int xad_accumulate_chain_gradients_f32(int strategy, std::size_t n, c
     // LDS table (at most 144 KiB): fp64 rows for every slot if they fit; if they fit in two
     // tables, the slots are dealt to two sets of blocks that each walk all threads (the inputs
     // are read twice, but ds_add_f64 is that much faster than ds_add_f32); otherwise fp32 rows
-    // for every slot if those fit; otherwise 4096 fp32 rows claimed on first use.
+    // for every slot if those fit; otherwise rows claimed on first use (2048 fp64 or 4096 fp32, below).
     constexpr std::size_t kTableBudget = 144 * 1024;
     std::size_t cells = static_cast<std::size_t>(num_slots) * kWidth;
     bool f32_table = strategy == XAD_ACCUMULATE_LDS_F32;
@@ -223,9 +223,15 @@ extern "C" int xad_accumulate_chain_gradients_f32(int strategy, std::size_t n, c
         cells = ((static_cast<std::size_t>(num_slots) + 1) / 2) * kWidth;
     }
     if (!f32_table && cells * sizeof(double) > kTableBudget) f32_table = true;
-    const std::size_t cell = f32_table ? sizeof(float) : sizeof(double);
+    std::size_t cell = f32_table ? sizeof(float) : sizeof(double);
     const bool direct = cells * cell <= kTableBudget;
-    a.capacity = direct ? static_cast<int>(cells / kWidth) : 4096;
+    // rows claimed on first use: up to 262 144 slots 2048 fp64 rows rather than 4096 fp32 ones (ds_add_f32 is
+    // 24x slower than ds_add_f64; beyond that the lower hit rate of the smaller table costs more than the
+    // slower adds, measured on Zipf(1.1) slots), unless the fp32 table was asked for by name
+    const bool tagged_f64 = !direct && staged && num_slots <= (1 << 18) && strategy != XAD_ACCUMULATE_LDS_F32 &&
+                            strategy != XAD_ACCUMULATE_LDS_LEAVES;
+    if (tagged_f64) cell = sizeof(double);
+    a.capacity = direct ? static_cast<int>(cells / kWidth) : (tagged_f64 ? 2048 : 4096);
     if (direct && staged && a.part_shift == 0) {
         // a small table is replicated: up to 16 copies within 48 KiB (two blocks per CU stay resident)
         const std::size_t copy_rows = static_cast<std::size_t>(BlockAccumulator<float, kWidth>::replica_rows(num_slots));
@@ -241,6 +247,16 @@ extern "C" int xad_accumulate_chain_gradients_f32(int strategy, std::size_t n, c
     }
     XAD_REQUIRE(lds <= kMaxLdsBytes, "%s: LDS table of %zu bytes does not fit", who, lds);
     const int per_cu = lds <= 72 * 1024 ? 2 : 1;  // two 1024-lane blocks fill a CU; 160 KiB of LDS hold two tables up to 72 KiB
+    if (a.spill_offset && tagged_f64) {
+        switch (strategy) {
+            case XAD_ACCUMULATE_WAVE_LDS:
+                return launch(accumulate_kernel<Strategy::WaveThenLds, 8, double, true>, a, lds, per_cu, stream);
+            case XAD_ACCUMULATE_WAVE_LDS_SHALLOW:
+                return launch(accumulate_kernel<Strategy::WaveThenLds, 2, double, true>, a, lds, per_cu, stream);
+            default:
+                return launch(accumulate_kernel<Strategy::LdsAtomics, 0, double, true>, a, lds, per_cu, stream);
+        }
+    }
     if (a.spill_offset) {
         switch (strategy) {
             case XAD_ACCUMULATE_WAVE_LDS:
