@@ -83,3 +83,34 @@ def shared_accumulation(blocks, threads):
     rc = load().xad_test_shared_accumulation(ctypes.c_int(blocks), ctypes.c_int(threads), out.ctypes.data_as(ctypes.c_void_p))
     assert rc == 0
     return out.reshape(blocks, 2)
+
+
+HOST_TESTER_PATH = os.path.join(HERE, "native", "libxad_tester_host.so")
+
+
+def run_tester_suite(device):
+    """Runs every gradient-tester call of the reference's tests plus the testers' self-checks:
+    in kernels (the HIP build) or on the calling thread (the g++ build).  Returns
+    (rows, self_check_bits), a row = (citation, name, cases, failures, worst error, on_device)."""
+    if device:
+        lib, fn_name = load(), "xad_test_tester_suite_device"
+    else:
+        if not os.path.exists(HOST_TESTER_PATH):
+            raise ImportError("tests/native/libxad_tester_host.so is not built; run `python tests/native/build.py`")
+        lib, fn_name = ctypes.CDLL(HOST_TESTER_PATH), "xad_test_tester_suite_host"
+        lib.xad_test_host_source_digest.restype = ctypes.c_char_p
+        load()  # checks the digest of the directory once ...
+        if lib.xad_test_host_source_digest() != _lib.xad_test_source_digest():  # ... which both libraries carry
+            raise ImportError("tests/native/libxad_tester_host.so is older than its sources; run `python tests/native/build.py`")
+    fn = getattr(lib, fn_name)
+    fn.argtypes = [ctypes.c_char_p, ctypes.c_size_t, ctypes.POINTER(ctypes.c_uint)]
+    text = ctypes.create_string_buffer(1 << 16)
+    bits = ctypes.c_uint(0)
+    count = fn(text, len(text), ctypes.byref(bits))
+    assert count >= 0, text.value.decode()
+    rows = []
+    for line in text.value.decode().splitlines():
+        citation, name, cases, failures, worst, on_device = line.split("|")
+        rows.append((citation, name, int(cases), int(failures), float(worst), on_device == "1"))
+    assert len(rows) == count
+    return rows, bits.value

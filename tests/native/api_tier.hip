@@ -9,6 +9,7 @@
 #include <cstring>
 
 #include "api_cases.cuh"
+#include "tester_suite.cuh"
 
 using namespace xyz_autodiff;
 
@@ -156,6 +157,11 @@ bool ok(hipError_t e) { return e == hipSuccess; }
 #define XAD_TEST_SOURCE_DIGEST ""
 #endif
 extern "C" const char* xad_test_source_digest(void) { return XAD_TEST_SOURCE_DIGEST; }
+
+// The gradient testers in this HIP translation unit: all cases of a tester call run in one kernel launch.
+extern "C" int xad_test_tester_suite_device(char* text, std::size_t capacity, unsigned* self_checks) {
+    return xad_suite::export_suite(text, capacity, self_checks);
+}
 
 extern "C" int xad_test_case_capacity(void) { return xad_test::kCaseCapacity; }
 

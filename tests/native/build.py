@@ -1,4 +1,5 @@
-"""Builds tests/native/libxad_api_tier.so (the API test tier) for gfx950 + host."""
+"""Builds tests/native/libxad_api_tier.so (the API test tier, hipcc: gfx950 + host pass) and
+tests/native/libxad_tester_host.so (the gradient testers compiled by g++ alone)."""
 import hashlib
 import os
 import subprocess
@@ -6,12 +7,13 @@ import subprocess
 HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(os.path.dirname(HERE))
 LIB = os.path.join(HERE, "libxad_api_tier.so")
+HOST_LIB = os.path.join(HERE, "libxad_tester_host.so")
 
 
 def source_digest():
     """SHA-256 over this directory's sources and the library headers they include."""
     h = hashlib.sha256()
-    files = [os.path.join(HERE, f) for f in os.listdir(HERE) if f.endswith((".hip", ".cuh"))]
+    files = [os.path.join(HERE, f) for f in os.listdir(HERE) if f.endswith((".hip", ".cuh", ".inc", ".cpp"))]
     for dirpath, _, names in os.walk(os.path.join(ROOT, "include")):
         files += [os.path.join(dirpath, f) for f in names if f.endswith((".cuh", ".h"))]
     for path in sorted(files):
@@ -34,6 +36,15 @@ def build():
     if proc.returncode != 0:
         noise = "is not a recognized feature for this target"
         raise RuntimeError("hipcc failed:\n" + "\n".join(l for l in proc.stderr.splitlines() if noise not in l))
+    host = [
+        os.environ.get("CXX", "g++"), "-std=c++20", "-O1", "-fPIC", "-shared", "-march=x86-64-v3",
+        "-I" + os.path.join(ROOT, "include"), "-I" + os.path.join(ROOT, "include", "mini-gaussian-splatting"),
+        "-DXAD_TEST_SOURCE_DIGEST=\"%s\"" % source_digest(),
+        os.path.join(HERE, "tester_host.cpp"), "-o", HOST_LIB,
+    ]
+    proc = subprocess.run(host, capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError("g++ failed:\n" + proc.stderr)
     return LIB
 
 
