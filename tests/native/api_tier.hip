@@ -10,6 +10,7 @@
 
 #include "api_cases.cuh"
 #include "tester_suite.cuh"
+#include "concept_checks.cuh"
 
 using namespace xyz_autodiff;
 
