@@ -114,10 +114,12 @@ def test_device_draw_matches_host_draw(gpu, oracle):
         np.testing.assert_allclose(hist[e], want, rtol=1e-12)
 
 
-def test_sgd_trajectory_matches_oracle(gpu, oracle):
+# the reference batch, a batch smaller than one launch grid, and one of most of the data set
+@pytest.mark.parametrize("batch,epochs", [(8192, 300), (1000, 50), (70_000, 40)])
+def test_sgd_trajectory_matches_oracle(gpu, oracle, batch, epochs):
     import torch
 
-    total, batch, epochs = 100_000, 8192, 300
+    total = 100_000
     x1, x2, y = linreg.synthetic_data(total, seed=6)
     rows = np.concatenate([linreg.batch_rows(5, e, batch, total) for e in range(epochs)])
     want_p, want_hist = oracle.linreg_sgd(x1, x2, y, rows, linreg.INITIAL_PARAMS, batch, epochs, 1e-4, 1e-6)
@@ -126,7 +128,7 @@ def test_sgd_trajectory_matches_oracle(gpu, oracle):
     # summation order differs per step (1e-16 relative); the iteration contracts, so the difference stays small
     np.testing.assert_allclose(params.cpu().numpy(), want_p, rtol=1e-9, atol=1e-10)
     np.testing.assert_allclose(hist, want_hist, rtol=1e-9)
-    assert hist[-1] < 0.5 * hist[0]
+    assert hist[-1] < (0.5 if epochs >= 300 else 1.0) * hist[0]
 
 
 def test_sgd_reference_hyperparameters_converge(gpu):
