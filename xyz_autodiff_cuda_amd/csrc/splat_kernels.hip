@@ -341,44 +341,60 @@ __global__ void __launch_bounds__(kChunk) render_forward_kernel(
     }
 }
 
-// Sum of nine per-lane values over the wavefront, cheaper than nine separate
-// reductions.  v[0..7] go through a reduce-scatter: at each of the first three
-// steps a lane hands half of its values to its partner (lane ^ 1, ^ 2, ^ 4) and
-// adds the partner's copies of the half it keeps, so after 4 + 2 + 1 exchanges
-// lane l holds value l % 8 summed over its group of eight lanes; one rotation
-// by eight completes the row of 16.  v[8] takes the ordinary four row steps.
-// Result: in every row of 16 lanes, lane m < 8 holds the row's sum of v[m] and
-// lane 8 that of v[8]; the four rows are added by whoever reads them.
+// Sum of nine per-lane values over each row of 16 lanes, cheaper than nine separate
+// reductions.  v[0..7] go through a reduce-scatter: at each of three steps a lane
+// keeps half of its values, the half chosen by one bit of its lane number, and
+// adds the copies held by the partner lane that differs in that bit.  For bits 2
+// and 3 (partners 4 and 8 lanes away) the choice is made by the bank mask of the
+// DPP add itself: one instruction serves the lanes whose bit is clear, a second
+// one the others, and no select is needed.  Bit 0 takes the ordinary select and
+// quad swap; a last quad swap over bit 1 completes the row.  v[8] takes the
+// ordinary four row steps.
+// Result: lane l of a row holds the row's sum of v[reduced_index(l)].
+__device__ __forceinline__ int reduced_index(int lane) {
+    const int r = lane & 15;
+    return (r & 2) ? 8 : ((r & 1) << 2) | ((r >> 3) << 1) | ((r >> 2) & 1);
+}
+
 __device__ __forceinline__ float reduce_scatter9(const float (&v)[9], int lane) {
-    const bool b0 = lane & 1, b1 = lane & 2, b2 = lane & 4;
-    float w[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const float keep = b0 ? v[2 * i + 1] : v[2 * i];
-        const float send = b0 ? v[2 * i] : v[2 * i + 1];
-        w[i] = keep + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, send), 0xB1, 0xF, 0xF, true));
-    }
-    float u[2];
-#pragma unroll
-    for (int i = 0; i < 2; ++i) {
-        const float keep = b1 ? w[2 * i + 1] : w[2 * i];
-        const float send = b1 ? w[2 * i] : w[2 * i + 1];
-        u[i] = keep + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, send), 0x4E, 0xF, 0xF, true));
-    }
-    const float keep = b2 ? u[1] : u[0];
-    const float send = b2 ? u[0] : u[1];
-    // lane ^ 4: a shift by four towards lower lanes feeds banks 0 and 2, towards higher lanes banks 1 and 3
-    int other = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, send), 0x104, 0xF, 0x5, false);   // row_shl:4
-    other = __builtin_amdgcn_update_dpp(other, __builtin_bit_cast(int, send), 0x114, 0xF, 0xA, false);    // row_shr:4
-    float t = keep + __builtin_bit_cast(float, other);
-    t = accumulate::wave::dpp_add<0x128>(t);  // row_ror:8
+    // bit 2: banks 0 and 2 (lanes 0-3, 8-11 of a row) keep the even value and read lane + 4,
+    // banks 1 and 3 keep the odd one and read lane - 4.  The leading wait covers the two idle
+    // cycles a DPP read needs after a vector write of the same register.
+    float w0, w1, w2, w3;
+    asm volatile(
+        "s_nop 1\n\t"
+        "v_add_f32_dpp %0, %4, %4 row_shl:4 row_mask:0xf bank_mask:0x5\n\t"
+        "v_add_f32_dpp %0, %5, %5 row_shr:4 row_mask:0xf bank_mask:0xa\n\t"
+        "v_add_f32_dpp %1, %6, %6 row_shl:4 row_mask:0xf bank_mask:0x5\n\t"
+        "v_add_f32_dpp %1, %7, %7 row_shr:4 row_mask:0xf bank_mask:0xa\n\t"
+        "v_add_f32_dpp %2, %8, %8 row_shl:4 row_mask:0xf bank_mask:0x5\n\t"
+        "v_add_f32_dpp %2, %9, %9 row_shr:4 row_mask:0xf bank_mask:0xa\n\t"
+        "v_add_f32_dpp %3, %10, %10 row_shl:4 row_mask:0xf bank_mask:0x5\n\t"
+        "v_add_f32_dpp %3, %11, %11 row_shr:4 row_mask:0xf bank_mask:0xa"
+        : "=&v"(w0), "=&v"(w1), "=&v"(w2), "=&v"(w3)
+        : "v"(v[0]), "v"(v[1]), "v"(v[2]), "v"(v[3]), "v"(v[4]), "v"(v[5]), "v"(v[6]), "v"(v[7]));
+    // bit 3: banks 0 and 1 (lanes 0-7) keep the even value, banks 2 and 3 the odd one; the partner is 8 lanes round the row
+    float u0, u1;
+    asm volatile(
+        "s_nop 1\n\t"
+        "v_add_f32_dpp %0, %2, %2 row_ror:8 row_mask:0xf bank_mask:0x3\n\t"
+        "v_add_f32_dpp %0, %3, %3 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+        "v_add_f32_dpp %1, %4, %4 row_ror:8 row_mask:0xf bank_mask:0x3\n\t"
+        "v_add_f32_dpp %1, %5, %5 row_ror:8 row_mask:0xf bank_mask:0xc"
+        : "=&v"(u0), "=&v"(u1)
+        : "v"(w0), "v"(w1), "v"(w2), "v"(w3));
+    const bool b0 = lane & 1;
+    const float keep = b0 ? u1 : u0;
+    const float send = b0 ? u0 : u1;
+    float t = keep + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, send), 0xB1, 0xF, 0xF, true));
+    t = accumulate::wave::dpp_add<0x4E>(t);  // bit 1
 
     float x = v[8];
     x = accumulate::wave::dpp_add<0xB1>(x);
     x = accumulate::wave::dpp_add<0x4E>(x);
     x = accumulate::wave::dpp_add<0x141>(x);
     x = accumulate::wave::dpp_add<0x140>(x);
-    return (lane & 8) ? x : t;
+    return (lane & 2) ? x : t;
 }
 
 // Compositing backward.  Lists are walked back to front.  For every Gaussian
@@ -389,7 +405,7 @@ __device__ __forceinline__ float reduce_scatter9(const float (&v)[9], int lane) 
 // (the Mahalanobis backward rule, d centre = -g_q (2a dx + 2b dy, 2b dx + 2c dy),
 // d inv = g_q (dx^2, 2 dx dy, dy^2), is linear in those sums, so it is applied
 // once per Gaussian instead of once per pixel).  The nine values are reduced
-// over the wavefront by reduce_scatter9 and parked in LDS; after every kPark
+// over each row of 16 lanes by reduce_scatter9 and parked in LDS; after every kPark
 // list entries lane j finishes entry j of the group, and the group's record
 // gradients are added to the global accumulator with consecutive lanes on
 // consecutive fields of consecutive entries: one atomic per (tile, Gaussian,
@@ -448,6 +464,9 @@ __global__ void __launch_bounds__(kChunk) render_backward_kernel(
     if (deepest == 0) return;
     const std::uint32_t first = range_begin[tile];
     const float px0 = static_cast<float>(x0);
+    // which of the nine row sums this lane ends up with; eight lanes and one more per row park theirs
+    const int park_index = reduced_index(lane);
+    const bool parks = !(lane & 2) || (lane & 15) == 2;
 
     for (std::uint32_t chunk = (deepest + kChunk - 1) / kChunk; chunk-- > 0;) {
         const std::uint32_t chunk_first = chunk * kChunk;
@@ -507,7 +526,7 @@ __global__ void __launch_bounds__(kChunk) render_backward_kernel(
                 const float sy = dy * m0;
                 const float v[9] = {sx, sy, ::fmaf(dx0, sx + m1, m2), dy * sx, dy * sy, colour[0], colour[1], colour[2], m0};
                 const float mine = reduce_scatter9(v, lane);
-                if ((lane & 15) < 9) parked[j - group_first][lane >> 4][lane & 15] = mine;
+                if (parks) parked[j - group_first][lane >> 4][park_index] = mine;
             }
             const int members = group_end - group_first;
             __syncthreads();
