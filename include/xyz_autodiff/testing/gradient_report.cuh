@@ -98,6 +98,18 @@ inline double min_abs_rel(double analytic, double numeric, double reference, dou
     return diff < rel ? diff : rel;  // a NaN diff makes the comparison false and returns the NaN rel
 }
 
+}  // namespace detail
+
+// The testers' error measure for one gradient element: min(|a - n|, |a - n| / (|a| + 1e-15))
+// (unary_gradient_tester.cuh:27-32 of the reference, same name).
+template <typename T>
+inline T compute_error_min(T analytical, T numerical) {
+    return static_cast<T>(detail::min_abs_rel(static_cast<double>(analytical), static_cast<double>(numerical),
+                                              static_cast<double>(analytical), 1e-15));
+}
+
+namespace detail {
+
 inline std::string describe(std::size_t test_case, const std::string& element, double analytic, double numeric, double error) {
     char text[256];
     std::snprintf(text, sizeof text, "test case %zu, %s: analytical=%.12g, numerical=%.12g, error_min=%.3g", test_case,

@@ -240,7 +240,8 @@ inline std::string describe(const std::vector<Entry>& entries) {
 //   2  a missing operand gradient is reported, on that operand only   3  a tolerance above 1e-5 is refused, nothing runs
 //   4  a negative tolerance is refused                                5  an inconsistent network fails test_single_case
 //   6  ... and test_network                                           7  a correct network passes test_single_case
-//   8  a logic instance with another constant is used by test_logic   9  zero cases is an empty, passing report
+//   8  a logic instance with another constant is used by test_logic   9  zero cases is an empty, passing report;
+//                                                                      compute_error_min is min(absolute, relative)
 inline unsigned run_self_checks() {
     unsigned ok = 0;
     const std::size_t before = testing::failure_count();
@@ -272,7 +273,10 @@ inline unsigned run_self_checks() {
         AddConstantTestLogic<double>(-40.0), "AddConstantTestLogic(-40)", 20, 1e-5, 1e-6, -1.0, 1.0);
     if (shifted && shifted.cases == 20) ok |= 1u << 8;
     const auto none = testing::UnaryGradientTester<op::ExpLogic<2>, 2, 2>::test_custom("no cases", 0, 1e-5, 1e-6);
-    if (none && none.cases == 0 && none.failures == 0) ok |= 1u << 9;
+    if (none && none.cases == 0 && none.failures == 0 && testing::compute_error_min(0.5, 0.75) == 0.25 &&  // absolute
+        testing::detail::absolute(testing::compute_error_min(8.0, 10.0) - 0.25) < 1e-12 &&  // relative
+        testing::compute_error_min(4.0f, 4.0f) == 0.0f)
+        ok |= 1u << 9;
     return ok;
 }
 
