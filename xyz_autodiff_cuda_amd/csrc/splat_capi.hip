@@ -45,6 +45,7 @@ struct xad_splat_context {
     static constexpr int kStages = 7;  // project, scan+emit, sort, ranges, render fwd, render bwd, parameter bwd
     hipEvent_t marks[kStages + 1] = {};
     float stage_ms[kStages] = {};
+    hipEvent_t count_ready = nullptr;  // the read-back of the pair count has arrived
 };
 
 namespace {
@@ -91,13 +92,24 @@ int order_by_depth(xad_splat_context* c, const float* depth, hipStream_t s) {
     return XAD_OK;
 }
 
-// Places the pairs: scan of the tile counts in depth order.  Reads back the number of pairs
-// (which sizes the sort) and the depth-changed flag: the one synchronisation of a step.
-int place_pairs(xad_splat_context* c, hipStream_t s) {
+int emit(xad_splat_context* c, hipStream_t s) {
+    std::uint32_t* depth_changed = c->offsets + c->G + 1;
+    return launch_emit(s, c->G, c->by_depth, c->rects, c->offsets, c->tiles_x, c->wide_keys, c->keys, c->ids, c->capacity,
+                       c->range_begin, c->tiles * 2, depth_changed);
+}
+
+// Places the pairs (scan of the tile counts in depth order) and emits them.  The number of pairs,
+// which sizes the sort, and the depth-changed flag are read back: the one wait of a step.  The
+// emission is queued before that wait, so it runs while the host is woken: it needs the offsets,
+// not the count, and never writes past the capacity.  (The copy that reads the flag is ahead of
+// the emission, which resets it, in the stream.)
+int place_and_emit(xad_splat_context* c, hipStream_t s) {
     if (int st = launch_permute_counts(s, c->G, c->by_depth, c->counts, c->counts_by_depth)) return st;
     if (int st = exclusive_scan_counts(s, c->scan_temp, c->scan_bytes, c->counts_by_depth, c->offsets, c->G)) return st;
     XAD_HIP_TRY(hipMemcpyAsync(c->host_pairs, c->offsets + c->G, 2 * sizeof(std::uint32_t), hipMemcpyDeviceToHost, s));
-    XAD_HIP_TRY(hipStreamSynchronize(s));
+    XAD_HIP_TRY(hipEventRecord(c->count_ready, s));
+    if (int st = emit(c, s)) return st;
+    XAD_HIP_TRY(hipEventSynchronize(c->count_ready));
     c->pairs = c->host_pairs[0];
     return XAD_OK;
 }
@@ -111,26 +123,25 @@ int bin(xad_splat_context* c, const float* params, const float* depth, hipStream
     const bool had_order = c->order_valid;
     if (!had_order)
         if (int st = order_by_depth(c, depth, s)) return st;
-    std::uint32_t* depth_changed = c->offsets + c->G + 1;  // zero at creation, reset by every emit
+    std::uint32_t* depth_changed = c->offsets + c->G + 1;  // zero at creation, reset by every emission
     if (int st = launch_project(s, c->G, params, depth, c->ordered_depth, depth_changed, c->width, c->height, c->records,
                                 c->rects, c->counts, c->record_grads, c->loss))
         return st;
     mark(c, 1, s);
     // The order of the previous call is used on the assumption that the depths are the same; the
     // flag read back with the pair count says whether they were, and if not the placement is redone.
-    if (int st = place_pairs(c, s)) return st;
+    if (int st = place_and_emit(c, s)) return st;
     if (had_order && c->host_pairs[1] != 0) {
         if (int st = order_by_depth(c, depth, s)) return st;
-        if (int st = place_pairs(c, s)) return st;
+        if (int st = place_and_emit(c, s)) return st;
     }
     if (c->pairs > c->capacity) {
+        // the emission above stopped at the old capacity; hipFree waits for it before the buffers go
         const std::uint64_t want = static_cast<std::uint64_t>(c->pairs) + c->pairs / 4 + 1024;
         XAD_REQUIRE(want < 0xffffffffull, "splat: %u pairs exceed the 32-bit pair index", c->pairs);
         if (int st = allocate_pair_buffers(c, static_cast<std::uint32_t>(want))) return st;
+        if (int st = emit(c, s)) return st;
     }
-    if (int st = launch_emit(s, c->G, c->by_depth, c->rects, c->offsets, c->tiles_x, c->wide_keys, c->keys, c->ids,
-                             c->capacity, c->range_begin, c->tiles * 2, depth_changed))
-        return st;
     mark(c, 2, s);
     if (int st = sort_pairs(s, c->sort_temp, c->sort_bytes, c->wide_keys, c->keys, c->keys_sorted, c->ids, c->ids_sorted,
                             c->pairs, c->key_bits))
@@ -220,6 +231,8 @@ extern "C" int xad_splat_create(int width, int height, int num_gaussians, std::s
     }
     for (auto& e : c->marks)
         if (st == XAD_OK && hipEventCreate(&e) != hipSuccess) st = xad::fail(XAD_ERR_HIP, "%s: hipEventCreate failed", who);
+    if (st == XAD_OK && hipEventCreateWithFlags(&c->count_ready, hipEventDisableTiming) != hipSuccess)
+        st = xad::fail(XAD_ERR_HIP, "%s: hipEventCreate failed", who);
     if (st != XAD_OK) {
         xad_splat_destroy(c);
         return st;
@@ -252,6 +265,7 @@ extern "C" void xad_splat_destroy(xad_splat_context* c) {
     if (c->host_loss) (void)hipHostFree(c->host_loss);
     for (auto& e : c->marks)
         if (e) (void)hipEventDestroy(e);
+    if (c->count_ready) (void)hipEventDestroy(c->count_ready);
     delete c;
 }
 
