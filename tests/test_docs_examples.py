@@ -23,3 +23,21 @@ def test_integration_example_compiles_for_gfx950(tmp_path):
            str(tmp_path / "example.o")]
     proc = subprocess.run(cmd, capture_output=True, text=True)
     assert proc.returncode == 0, proc.stderr
+
+
+def test_integration_host_stub_compiles(tmp_path):
+    """The C++ stubs of INTEGRATION.md against include/xad_capi.h (syntax and types only)."""
+    gxx = shutil.which("g++")
+    hip_include = "/opt/rocm/include"
+    if not gxx or not os.path.exists(os.path.join(hip_include, "hip", "hip_runtime_api.h")):
+        pytest.skip("g++ or the HIP headers are not installed")
+    text = open(os.path.join(ROOT, "INTEGRATION.md")).read()
+    block = re.search(r"```cpp\n(// replaces launch_gaussian_splatting.*?)```", text, re.S)
+    assert block, "the host stub is missing from INTEGRATION.md"
+    prelude = ("#include <cstddef>\n#include <stdexcept>\n#include <hip/hip_runtime_api.h>\n"
+               "static float lr_pos = 1e-2f, lr_scale = 1e-2f, lr_rot = 1e-2f, lr_col = 1e-2f, lr_opacity = 1e-2f;\n")
+    src = tmp_path / "stub.cpp"
+    src.write_text(prelude + block.group(1))
+    cmd = [gxx, "-std=c++17", "-fsyntax-only", "-D__HIP_PLATFORM_AMD__", "-I" + hip_include, "-I" + os.path.join(ROOT, "include"), str(src)]
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    assert proc.returncode == 0, proc.stderr
