@@ -145,3 +145,41 @@ def test_full_size_finite_differences_property(gpu, oracle):
     sample = [t[idx].cpu().numpy() for t in ins]
     got = np.stack([o[idx].cpu().numpy() for o in outs])
     _check(got, sample, oracle)
+
+
+def test_more_than_two_to_the_32_problems(gpu, oracle):
+    """13 arrays of 2^32 + 4099 floats (223 GB) fit the 288 GB of one MI355X: indices beyond 32 bits and
+    the seams between the launches such a call is split into.  Skipped where that much memory is not free."""
+    import torch
+
+    from xyz_autodiff_cuda_amd import chain, rng
+
+    n = (1 << 32) + 4099
+    torch.cuda.empty_cache()
+    free, _ = torch.cuda.mem_get_info(gpu)
+    if free < 13 * 4 * n + (4 << 30):
+        pytest.skip("needs %.0f GB of free device memory, %.0f GB are free" % (13 * 4 * n / 1e9, free / 1e9))
+    ins = [torch.empty(n, dtype=torch.float32, device=gpu) for _ in range(6)]
+    rng.chain_inputs_(ins, seed=99)
+    outs = [torch.empty(n, dtype=torch.float32, device=gpu) for _ in range(7)]
+    # what a lane that is never launched would leave behind, at the places looked at below
+    seam = (1 << 32) - (1 << 20)  # first problem of the second launch
+    windows = [(0, 4096), ((1 << 31) - 2048, (1 << 31) + 2048), (seam - 2048, seam + 2048), ((1 << 32) - 2048, n)]
+    for lo, hi in windows:
+        for o in outs:
+            o[lo:hi] = float("nan")
+    chain.forward_backward(ins, outs)
+    torch.cuda.synchronize()
+    for lo, hi in windows:
+        sample = [t[lo:hi].cpu().numpy() for t in ins]
+        got = np.stack([o[lo:hi].cpu().numpy() for o in outs])
+        _check(got, sample, oracle)
+    # every problem: the identity d w / d o = w (1 - sigmoid(o)), in pieces that fit beside the arrays
+    piece = 1 << 28
+    for lo in range(0, n, piece):
+        hi = min(n, lo + piece)
+        w, d_o = outs[0][lo:hi].double(), outs[4][lo:hi].double()
+        ident = (d_o - w * (1 - torch.sigmoid(ins[3][lo:hi].double()))).abs().max()
+        assert float(ident) < 1e-6, (lo, float(ident))
+    del ins, outs
+    torch.cuda.empty_cache()

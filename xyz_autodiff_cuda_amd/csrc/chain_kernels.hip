@@ -157,20 +157,22 @@ int launch_chain(std::size_t n, const ChainBuffers& buf, int problems_per_lane, 
         XAD_REQUIRE(buf.out[a], "%s: output array %d is null", who, a);
         vector_ok = vector_ok && xad::aligned16(buf.out[a]);
     }
-    XAD_REQUIRE(n <= 0x7fffffffull * 64, "%s: n = %zu exceeds the grid limit", who, n);
-
+    // a launch holds fewer than 2^32 lanes; larger arrays (they fit: 13 arrays of 2^32 floats are 223 GB) take several
+    constexpr std::size_t kLaunchLanes = (std::size_t(1) << 32) - (std::size_t(1) << 20);
     hipStream_t s = xad::as_stream(stream);
     const std::size_t groups = vector_ok ? n / 4 : 0;
+    XAD_REQUIRE(groups <= kLaunchLanes, "%s: n = %zu exceeds one launch of the four-problems-per-lane mapping", who, n);
     if (groups) {
         hipLaunchKernelGGL(chain_quad_kernel, dim3(xad::blocks_for(groups, kQuadBlock)), dim3(kQuadBlock), 0, s, buf,
                            groups);
         XAD_HIP_TRY(hipGetLastError());
     }
-    const std::size_t done = groups * 4;
-    if (done < n) {
-        hipLaunchKernelGGL(chain_single_kernel<StorePolicy::WriteThrough>, dim3(xad::blocks_for(n - done, kSingleBlock)),
-                           dim3(kSingleBlock), 0, s, buf, done, n);
+    for (std::size_t done = groups * 4; done < n;) {
+        const std::size_t part = std::min(n - done, kLaunchLanes);
+        hipLaunchKernelGGL(chain_single_kernel<StorePolicy::WriteThrough>, dim3(xad::blocks_for(part, kSingleBlock)),
+                           dim3(kSingleBlock), 0, s, buf, done, done + part);
         XAD_HIP_TRY(hipGetLastError());
+        done += part;
     }
     return XAD_OK;
 }
