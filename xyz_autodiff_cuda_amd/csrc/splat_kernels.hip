@@ -285,7 +285,9 @@ __global__ void __launch_bounds__(kChunk) render_forward_kernel(
     const float py = static_cast<float>(y);
     const float px0 = static_cast<float>(x0);
 
-    const std::uint32_t first = range_begin[tile], last = range_end[tile];
+    // the same for every lane: said so, which keeps the loop counters in scalar registers
+    const std::uint32_t first = __builtin_amdgcn_readfirstlane(range_begin[tile]);
+    const std::uint32_t last = __builtin_amdgcn_readfirstlane(range_end[tile]);
     float T[kLanePixels], red[kLanePixels], green[kLanePixels], blue[kLanePixels];
     std::uint32_t used[kLanePixels];
 #pragma unroll
@@ -300,7 +302,7 @@ __global__ void __launch_bounds__(kChunk) render_forward_kernel(
         __syncthreads();
         if (base + lane < last) staged[lane] = stage_record(records, sorted_ids[base + lane]);
         __syncthreads();
-        const int count = static_cast<int>(last - base < kChunk ? last - base : kChunk);
+        const int count = __builtin_amdgcn_readfirstlane(static_cast<int>(last - base < kChunk ? last - base : kChunk));
         for (int j = 0; j < count; ++j) {
             const Staged r = staged[j];
             // exponent of the falloff as a polynomial in dx: (a_s dx + e) dx + f
