@@ -18,7 +18,9 @@
  *   Adam (oracle_adam.c) and the renderer (oracle_splat.inc): the reference's tests
  *       hold no expected values for either (parity with the reference is unpinned
  *       in that sense); pinned by closed forms, an fp64 recurrence, a brute-force
- *       renderer, invariance to listing order and central differences of the loss.
+ *       renderer, invariance to listing order, central differences of the loss, and
+ *       an independently written renderer whose gradients come from reverse-mode
+ *       autodiff (image, loss and all nine gradients of a single-tile scene).
  *
  * Built twice over by the preprocessor: every op exists as name_f32 (float
  * arithmetic with the float libm routines, i.e. what the reference computes in

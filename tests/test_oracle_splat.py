@@ -166,3 +166,55 @@ def test_adam_many_steps_match_fp64_recurrence(oracle):
         vd = b2 * vd + (1 - b2) * g.astype(np.float64) ** 2
         pd -= lr * np.sqrt(1 - b2 ** t) / (1 - b1 ** t) * md / (np.sqrt(vd) + eps)
     assert np.allclose(p, pd, atol=2e-5)
+
+
+def test_single_tile_scene_matches_an_independent_autograd_renderer(oracle):
+    """An independent statement of the whole step: covariance R diag(s^2) R^T inverted by a library routine,
+    alpha = min(0.99, sigmoid(o) exp(-d^T Sigma^-1 d / 2)), (depth, index) order, front-to-back compositing
+    that stops a pixel before the first Gaussian met with T < 1e-4, loss = sum of squared differences;
+    its gradients come from reverse-mode autodiff of that code, not from hand-written rules.  One 16 x 16
+    tile with every centre inside it, so binning plays no part.  Rotated anisotropic Gaussians: a transposed
+    rotation, a wrong sign of the off-diagonal term or a swapped axis would show here."""
+    import torch
+
+    W = H = 16
+    G = 14
+    params, depth = random_scene(G, W, H, 21, scale_px=(1.0, 6.0))
+    # three wide, nearly opaque Gaussians in front of the rest, close together: where they overlap alpha clamps
+    # and T falls to 1e-6, so the pixels there stop before the fourth
+    params[8, :3] = 9.0
+    params[2:4, :3] = np.log(7.0)
+    params[0, :3] = (7.0, 8.5, 9.0)
+    params[1, :3] = (8.0, 7.5, 8.5)
+    depth[:3] = (0.01, 0.02, 0.03)
+    target = np.random.default_rng(22).uniform(0, 1, (H, W, 3)).astype(np.float32)
+    out = oracle.splat_step(W, H, params, depth, target, np.float64)
+
+    p = torch.tensor(params.astype(np.float64), requires_grad=True)
+    cx, cy, lsx, lsy, theta, red, green, blue, opacity = p
+    c, s = torch.cos(theta), torch.sin(theta)
+    rot = torch.stack([torch.stack([c, -s], -1), torch.stack([s, c], -1)], -2)  # (G, 2, 2)
+    scale2 = torch.diag_embed(torch.exp(torch.stack([lsx, lsy], -1)) ** 2)
+    inverse = torch.linalg.inv(rot @ scale2 @ rot.transpose(-1, -2))
+    ys, xs = torch.meshgrid(torch.arange(H, dtype=torch.float64), torch.arange(W, dtype=torch.float64), indexing="ij")
+    d = torch.stack([xs[None] - cx[:, None, None], ys[None] - cy[:, None, None]], -1)  # (G, H, W, 2)
+    q = torch.einsum("ghwi,gij,ghwj->ghw", d, inverse, d)
+    alpha = torch.minimum(torch.sigmoid(opacity)[:, None, None] * torch.exp(-0.5 * q), torch.tensor(0.99, dtype=torch.float64))
+    colour = torch.stack([red, green, blue], -1)
+    order = sorted(range(G), key=lambda g: (float(depth[g]), g))
+    T = torch.ones(H, W, dtype=torch.float64)
+    image = torch.zeros(H, W, 3, dtype=torch.float64)
+    stopped = torch.zeros(H, W, dtype=torch.bool)
+    for g in order:
+        stopped = stopped | (T.detach() < 1e-4)
+        a = torch.where(stopped, torch.zeros_like(T), alpha[g])
+        image = image + (T * a)[..., None] * colour[g]
+        T = T * (1 - a)
+    assert bool(stopped.any()) and bool((alpha >= 0.99).any()), "the scene must exercise the cut-off and the clamp"
+    loss = ((image - torch.tensor(target.astype(np.float64))) ** 2).sum()
+    loss.backward()
+    assert np.allclose(out["image"], image.detach().numpy(), rtol=1e-11, atol=1e-14)
+    assert np.isclose(out["loss"], float(loss.detach()), rtol=1e-12)
+    want = p.grad.numpy()
+    scale = np.abs(want).max(axis=1, keepdims=True)
+    assert np.all(np.abs(out["grads"] - want) <= 1e-9 * scale + 1e-14), np.abs(out["grads"] - want).max()
