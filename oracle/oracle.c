@@ -10,7 +10,8 @@
  *       differences in fp64, the guards and special cases of the reference's op tests;
  *   chain (oracle_chain_*)         the reference's own evaluation of the graph at the
  *       points of tests/golden/chain_reference_vector.json, a closed form without a
- *       matrix inverse, central differences;
+ *       matrix inverse, reverse-mode autodiff of an independent statement, central
+ *       differences;
  *   accumulation sums              a bincount formulation and the reference's exact
  *       counting pattern (tests/test_parallel_gradient_accumulation.cu:94-99);
  *   least squares (oracle_linreg.c) hand-computed gradients at the reference's test

@@ -90,3 +90,24 @@ def test_fp32_error_is_conditioning_not_a_bug(oracle):
     assert e[0].max() < 1e-5  # the value itself
     assert e[:, kappa <= 7.4].max(initial=0.0) < 1e-5  # e^(2*1): more than half of all problems
     assert (e / np.maximum(1.0, kappa)).max() < 1e-5
+
+
+def test_fp64_matches_reverse_mode_autodiff_of_an_independent_statement(oracle):
+    """w = sigmoid(o) exp(-p^T Sigma^-1 p / 2) with Sigma = R(theta) diag(exp(s))^2 R(theta)^T inverted by a
+    library routine; the six gradients by PyTorch's autograd.  Nothing of the oracle's rules is retyped here."""
+    import torch
+
+    inputs = [np.asarray(a, np.float64) for a in chain_inputs(500, seed=77)]
+    got = oracle.chain_soa(inputs, np.float64)
+    sx, sy, theta, o, px, py = (torch.tensor(a, requires_grad=True) for a in inputs)
+    c, s = torch.cos(theta), torch.sin(theta)
+    rot = torch.stack([torch.stack([c, -s], -1), torch.stack([s, c], -1)], -2)
+    sigma = rot @ torch.diag_embed(torch.exp(torch.stack([sx, sy], -1)) ** 2) @ rot.transpose(-1, -2)
+    p = torch.stack([px, py], -1)
+    q = torch.einsum("ni,nij,nj->n", p, torch.linalg.inv(sigma), p)
+    w = torch.sigmoid(o) * torch.exp(-0.5 * q)
+    w.sum().backward()
+    want = np.stack([w.detach().numpy()] + [t.grad.numpy() for t in (sx, sy, theta, o, px, py)])
+    # the inverse of an ill-conditioned Sigma carries cond(Sigma) ulps in either evaluation
+    kappa = np.exp(2.0 * np.abs(inputs[0] - inputs[1]))
+    assert (abs_or_rel(got, want) / kappa).max() < 1e-12
