@@ -7,7 +7,9 @@
  * What pins each part (tests/test_oracle_*.py, tests/test_accumulate_oracle.py);
  * no function here is left unpinned:
  *   per-op rules (oracle_ops.inc)  formulas written independently in numpy, central
- *       differences in fp64, the guards and special cases of the reference's op tests;
+ *       differences in fp64, reverse-mode autodiff of every op written once more as
+ *       a differentiable expression, the guards and special cases of the reference's
+ *       op tests;
  *   chain (oracle_chain_*)         the reference's own evaluation of the graph at the
  *       points of tests/golden/chain_reference_vector.json, a closed form without a
  *       matrix inverse, reverse-mode autodiff of an independent statement, central
