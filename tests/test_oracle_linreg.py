@@ -133,3 +133,18 @@ def test_sgd_recovers_true_parameters_without_noise(oracle):
     # a, b, c settle quickly; the offset d is the flat direction of this loss and is still on its way
     np.testing.assert_allclose(p[:3], linreg.TRUE_PARAMS[:3], atol=0.05)
     assert 0.1 < p[3] < linreg.TRUE_PARAMS[3] + 0.05
+
+
+def test_gradient_matches_reverse_mode_autodiff(oracle):
+    """The summed loss sum_i ((x1 - a)^2 + b (x2 - c)^2 + d - y)^2 differentiated by PyTorch's autograd."""
+    import torch
+
+    x1, x2, y = linreg.synthetic_data(3000, seed=12, noise=0.3)
+    for params in ([0.5, 1.5, -0.5, 0.2], [2.5, 1.8, -1.2, 0.5], [-3.0, 0.1, 4.0, -7.0]):
+        p = torch.tensor(params, dtype=torch.float64, requires_grad=True)
+        a, b, c, d = p
+        loss = (((torch.tensor(x1) - a) ** 2 + b * (torch.tensor(x2) - c) ** 2 + d - torch.tensor(y)) ** 2).sum()
+        loss.backward()
+        out = oracle.linreg_gradient(x1, x2, y, params)
+        np.testing.assert_allclose(out[:4], p.grad.numpy(), rtol=1e-11)
+        np.testing.assert_allclose(out[4], float(loss.detach()), rtol=1e-12)
