@@ -168,6 +168,27 @@ def test_adam_many_steps_match_fp64_recurrence(oracle):
     assert np.allclose(p, pd, atol=2e-5)
 
 
+def test_adam_many_steps_match_a_library_optimiser(oracle):
+    """torch.optim.Adam divides by sqrt(v / (1 - b2^t)) + eps, the rule here by (sqrt(v) + eps) / sqrt(1 - b2^t):
+    the same step once the library is given eps / sqrt(1 - b2^t).  An implementation nobody here wrote."""
+    import torch
+
+    r = np.random.default_rng(5)
+    p0 = r.normal(0, 1, 400).astype(np.float32)
+    p, m, v = p0.copy(), np.zeros_like(p0), np.zeros_like(p0)
+    lr, b1, b2, eps = 1e-2, 0.9, 0.999, 1e-8
+    tp = torch.tensor(p0.astype(np.float64), requires_grad=True)
+    opt = torch.optim.Adam([tp], lr=lr, betas=(b1, b2), eps=eps)
+    for t in range(1, 41):
+        g = r.normal(0, 1, 400).astype(np.float32)
+        g[::40] = 0.0
+        oracle.adam_step(p, g, m, v, lr, b1, b2, eps, t)
+        opt.param_groups[0]["eps"] = eps / np.sqrt(1 - b2 ** t)
+        tp.grad = torch.tensor(g.astype(np.float64))
+        opt.step()
+    assert np.allclose(p, tp.detach().numpy(), atol=2e-5)
+
+
 def test_single_tile_scene_matches_an_independent_autograd_renderer(oracle):
     """An independent statement of the whole step: covariance R diag(s^2) R^T inverted by a library routine,
     alpha = min(0.99, sigmoid(o) exp(-d^T Sigma^-1 d / 2)), (depth, index) order, front-to-back compositing
