@@ -435,6 +435,7 @@ def main():
         "outputs_finite": finite,
         "mapping_GBps": alt,
         "store_policy_GBps": store_policy,
+        "kernel_resources": chain.kernel_resources(),
     }
     record["accumulate"] = accumulate_report(ins, args.seed, with_oracle=not args.no_cpu)
     if not args.no_cpu:

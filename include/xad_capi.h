@@ -359,6 +359,14 @@ int xad_host_linreg_gradient_f64(size_t n, size_t total,
  */
 int xad_probe_lds_atomic_cycles(int element, int pattern, double* cycles_per_instruction);
 
+/* Resources of the default kernel of xad_chain_forward_backward_f32 as the loaded
+ * code object and the current device report them: vector registers per lane,
+ * scratch (spill) bytes per lane, static LDS bytes per block, lanes per block, and
+ * how many such blocks one compute unit holds at once.  out[5] in that order.
+ * No counterpart in the reference.
+ */
+int xad_chain_kernel_resources(int* out);
+
 /* Hardware probe behind the default kernel of xad_chain_forward_backward_f32: the
  * same kernel (one problem per lane, non-temporal loads) with its seven results
  * stored as 0 write-through stores (relaxed atomic stores at agent scope, the

@@ -32,6 +32,10 @@ def load():
     if _lib is None:
         if not os.path.exists(LIB_PATH):
             raise ImportError("tests/native/libxad_api_tier.so is not built; run `python tests/native/build.py`")
+        try:  # PyTorch's HIP runtime first, so that the process has one (see xyz_autodiff_cuda_amd/_lib.py)
+            import torch  # noqa: F401
+        except ImportError:
+            pass
         lib = ctypes.CDLL(LIB_PATH)
         lib.xad_test_source_digest.restype = ctypes.c_char_p
         import importlib.util

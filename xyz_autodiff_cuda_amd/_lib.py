@@ -67,6 +67,7 @@ SIGNATURES = {
     "xad_linreg_sgd_f64": [_sz, _vp, _vp, _vp, _vp, _int, _int, ctypes.c_double, ctypes.c_double, _u64, _vp, _vp],
     "xad_host_linreg_gradient_f64": [_sz, _sz, _vp, _vp, _vp, _vp, _vp, _vp],
     "xad_probe_chain_store_policy": [_int, _sz] + [_vp] * 13 + [_vp],
+    "xad_chain_kernel_resources": [_vp],
     "xad_probe_lds_atomic_cycles": [_int, _int, ctypes.POINTER(ctypes.c_double)],
     "xad_rng_zipf_i32": [_vp, _sz, _u64, _u64, _int, ctypes.c_double, _vp],
     "xad_rng_uniform_f32": [_vp, _sz, _u64, _u64, _flt, _flt, _vp],
@@ -87,6 +88,13 @@ def load():
         raise ImportError(
             "libxad_hip.so is not built (expected at %s); run `python -m xyz_autodiff_cuda_amd.build`" % LIB_PATH
         )
+    # PyTorch brings a HIP runtime of its own; whichever of the two libraries is loaded first decides which
+    # runtime the process uses.  With PyTorch first there is one runtime, the one that owns the tensors'
+    # memory; with this library first its kernels found no device once PyTorch had initialised its own.
+    try:
+        import torch  # noqa: F401
+    except ImportError:
+        pass
     lib = ctypes.CDLL(LIB_PATH)
     for name, argtypes in SIGNATURES.items():
         fn = getattr(lib, name)

@@ -78,6 +78,17 @@ def store_policy_probe(inputs, outputs, policy, stream=None):
     return outputs
 
 
+def kernel_resources():
+    """Registers, scratch, LDS and residency of the default kernel, as the loaded code object and the device report them."""
+    import ctypes
+
+    out = (ctypes.c_int * 5)()
+    _lib.check(_lib.load().xad_chain_kernel_resources(ctypes.cast(out, ctypes.c_void_p)), "xad_chain_kernel_resources")
+    vgprs, scratch, lds, lanes, blocks = list(out)
+    return {"vgprs_per_lane": vgprs, "scratch_bytes_per_lane": scratch, "lds_bytes_per_block": lds, "lanes_per_block": lanes,
+            "blocks_per_cu": blocks, "wavefronts_per_simd": blocks * lanes // 64 // 4}
+
+
 def host_forward_backward(inputs, dtype=np.float32, num_threads=0):
     """The same templates compiled for the host cores; numpy in, numpy out."""
     lib = _lib.load()

@@ -179,6 +179,21 @@ int launch_chain(std::size_t n, const ChainBuffers& buf, int problems_per_lane, 
 
 }  // namespace
 
+extern "C" int xad_chain_kernel_resources(int* out) {
+    XAD_REQUIRE(out, "xad_chain_kernel_resources: out is null");
+    const void* kernel = reinterpret_cast<const void*>(chain_single_kernel<StorePolicy::WriteThrough>);
+    hipFuncAttributes attr;
+    XAD_HIP_TRY(hipFuncGetAttributes(&attr, kernel));
+    int blocks_per_cu = 0;
+    XAD_HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&blocks_per_cu, kernel, static_cast<int>(kSingleBlock), 0));
+    out[0] = attr.numRegs;
+    out[1] = static_cast<int>(attr.localSizeBytes);
+    out[2] = static_cast<int>(attr.sharedSizeBytes);
+    out[3] = static_cast<int>(kSingleBlock);
+    out[4] = blocks_per_cu;
+    return XAD_OK;
+}
+
 extern "C" int xad_probe_chain_store_policy(int policy, std::size_t n, const float* sx, const float* sy,
                                             const float* theta, const float* o, const float* px, const float* py,
                                             float* w, float* d_sx, float* d_sy, float* d_theta, float* d_o,
