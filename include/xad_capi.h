@@ -342,6 +342,29 @@ int xad_linreg_gradient_f64(int strategy, size_t n, size_t total,
 int xad_linreg_sgd_f64(size_t total, const double* x1, const double* x2, const double* y,
                        double* params, int batch, int epochs, double lr_first, double lr_last,
                        uint64_t seed, double* loss_history, void* stream);
+/* xad_linreg_sgd_f64 for callers that cannot allocate device memory (code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  No
+ * counterpart in the reference.  Same arguments, same kernels and same results
+ * as xad_linreg_sgd_f64, with two differences:
+ *   - the gradient sums of a step live in a 256-byte array that is part of the
+ *     library's device image (one copy per device, held until the process ends)
+ *     instead of a buffer allocated and freed by the call; the call makes no
+ *     hipMalloc, hipFree or other allocating call and no host-device copy;
+ *   - it is asynchronous: it returns when the steps are queued on `stream`;
+ *     params and loss_history are final when the stream has run them.
+ * The scratch does not depend on total or batch; the one size a call bounds is
+ * the number of steps it queues (two launches each): epochs beyond
+ * XAD_LINREG_STATIC_MAX_EPOCHS are refused with XAD_ERR_INVALID_ARGUMENT.
+ * Every call on a device shares that device's array: calls whose work overlaps
+ * on one device (two streams, two host threads) race and give wrong sums; calls
+ * on one stream, or ordered by events, are fine, and each call clears the sums
+ * before its first step.  The first call on a device looks up the array's
+ * address (hipGetSymbolAddress); make it outside graph capture, e.g. with
+ * epochs = 0. */
+#define XAD_LINREG_STATIC_MAX_EPOCHS (1 << 20)
+int xad_linreg_sgd_f64_static(size_t total, const double* x1, const double* x2, const double* y,
+                              double* params, int batch, int epochs, double lr_first, double lr_last,
+                              uint64_t seed, double* loss_history, void* stream);
 /* Host cores: the same graph templates compiled for the CPU, one thread; all
  * pointers host. */
 int xad_host_linreg_gradient_f64(size_t n, size_t total,

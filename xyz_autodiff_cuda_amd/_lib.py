@@ -65,6 +65,7 @@ SIGNATURES = {
     "xad_trainer_load_checkpoint": [_vp, ctypes.c_char_p],
     "xad_linreg_gradient_f64": [_int, _sz, _sz, _vp, _vp, _vp, _vp, _vp, _vp, _vp],
     "xad_linreg_sgd_f64": [_sz, _vp, _vp, _vp, _vp, _int, _int, ctypes.c_double, ctypes.c_double, _u64, _vp, _vp],
+    "xad_linreg_sgd_f64_static": [_sz, _vp, _vp, _vp, _vp, _int, _int, ctypes.c_double, ctypes.c_double, _u64, _vp, _vp],
     "xad_host_linreg_gradient_f64": [_sz, _sz, _vp, _vp, _vp, _vp, _vp, _vp],
     "xad_probe_chain_store_policy": [_int, _sz] + [_vp] * 13 + [_vp],
     "xad_chain_kernel_resources": [_vp],

@@ -4,6 +4,7 @@
 // keeps parameters, gradient sums and the batch draw on the device.
 #include <cmath>
 #include <climits>
+#include <mutex>
 
 #include <xyz_autodiff/accumulate.cuh>
 
@@ -177,6 +178,62 @@ extern "C" int xad_linreg_gradient_f64(int strategy, size_t n, size_t total, con
     return launch_gradient(strategy, a, blocks, s);
 }
 
+namespace {
+
+// Queues `epochs` SGD steps on `s`; `sums` is kWidth doubles of device memory that
+// nothing else uses until the queued work has run.
+int queue_sgd(hipStream_t s, double* sums, std::size_t total, const double* x1, const double* x2, const double* y,
+              double* params, int batch, int epochs, double lr_first, double lr_last, std::uint64_t seed,
+              double* loss_history) {
+    unsigned blocks = 0;
+    if (int st = grid_for(static_cast<std::size_t>(batch), &blocks)) return st;
+    // the sums start from zero whatever an earlier run left in them (the update kernel clears them
+    // again after every step)
+    linreg_zero_kernel<<<1, 64, 0, s>>>(sums);
+    XAD_HIP_TRY(hipGetLastError());
+    const std::uint64_t key = xad_rng::stream_key(seed, 0);
+    const double decay = epochs > 0 ? std::log(lr_last / lr_first) / epochs : 0.0;
+    for (int e = 0; e < epochs; ++e) {
+        LinregArgs a{x1, x2, y, nullptr, params, sums, static_cast<std::size_t>(batch), total,
+                     key, static_cast<std::uint64_t>(e) * static_cast<std::uint64_t>(batch), true};
+        if (int st = launch_gradient(XAD_LINREG_WAVE_LDS, a, blocks, s)) return st;
+        linreg_update_kernel<<<1, 64, 0, s>>>(params, sums, lr_first * std::exp(decay * e), batch,
+                                              loss_history ? loss_history + e : nullptr);
+        XAD_HIP_TRY(hipGetLastError());
+    }
+    return XAD_OK;
+}
+
+// Gradient sums of xad_linreg_sgd_f64_static: one copy of this array per device, for the life of
+// the process.  kWidth doubles are used; the size is the alignment unit.
+constexpr int kScratchDoubles = 32;
+static __device__ __align__(256) double scratch[kScratchDoubles];
+static_assert(kWidth <= kScratchDoubles, "the sums must fit the static array");
+
+// Host code never passes `scratch` itself to a kernel: the name is a host-side handle, not a
+// device address.  The address is looked up once per device, with that device current.
+constexpr int kMaxDevices = 64;
+std::mutex scratch_lock;
+double* scratch_address[kMaxDevices] = {};
+
+int scratch_of_current_device(double** out) {
+    int dev = -1;
+    XAD_HIP_TRY(hipGetDevice(&dev));
+    XAD_REQUIRE(dev >= 0 && dev < kMaxDevices, "device %d is beyond the %d devices this entry point keeps scratch for", dev,
+                kMaxDevices);
+    std::lock_guard<std::mutex> guard(scratch_lock);
+    if (!scratch_address[dev]) {
+        void* p = nullptr;
+        XAD_HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        XAD_REQUIRE(p, "hipGetSymbolAddress returned a null address for the scratch array");
+        scratch_address[dev] = static_cast<double*>(p);
+    }
+    *out = scratch_address[dev];
+    return XAD_OK;
+}
+
+}  // namespace
+
 extern "C" int xad_linreg_sgd_f64(size_t total, const double* x1, const double* x2, const double* y, double* params,
                                   int batch, int epochs, double lr_first, double lr_last, uint64_t seed,
                                   double* loss_history, void* stream) {
@@ -186,30 +243,29 @@ extern "C" int xad_linreg_sgd_f64(size_t total, const double* x1, const double* 
     hipStream_t s = xad::as_stream(stream);
     double* sums = nullptr;
     XAD_HIP_TRY(hipMalloc(&sums, kWidth * sizeof(double)));
-    int status = XAD_OK;
-    unsigned blocks = 0;
-    status = grid_for(static_cast<std::size_t>(batch), &blocks);
-    if (status == XAD_OK) {
-        linreg_zero_kernel<<<1, 64, 0, s>>>(sums);
-        const std::uint64_t key = xad_rng::stream_key(seed, 0);
-        const double decay = std::log(lr_last / lr_first) / epochs;
-        for (int e = 0; e < epochs && status == XAD_OK; ++e) {
-            LinregArgs a{x1, x2, y, nullptr, params, sums, static_cast<std::size_t>(batch), total,
-                         key, static_cast<std::uint64_t>(e) * static_cast<std::uint64_t>(batch), true};
-            status = launch_gradient(XAD_LINREG_WAVE_LDS, a, blocks, s);
-            if (status != XAD_OK) break;
-            linreg_update_kernel<<<1, 64, 0, s>>>(params, sums, lr_first * std::exp(decay * e), batch,
-                                                  loss_history ? loss_history + e : nullptr);
-        }
-    }
-    const hipError_t launched = hipGetLastError();
+    const int status = queue_sgd(s, sums, total, x1, x2, y, params, batch, epochs, lr_first, lr_last, seed, loss_history);
     const hipError_t waited = hipStreamSynchronize(s);
     const hipError_t freed = hipFree(sums);
     if (status != XAD_OK) return status;
-    XAD_HIP_TRY(launched);
     XAD_HIP_TRY(waited);
     XAD_HIP_TRY(freed);
     return XAD_OK;
+}
+
+extern "C" int xad_linreg_sgd_f64_static(size_t total, const double* x1, const double* x2, const double* y,
+                                         double* params, int batch, int epochs, double lr_first, double lr_last,
+                                         uint64_t seed, double* loss_history, void* stream) {
+    const char* who = "xad_linreg_sgd_f64_static";
+    XAD_REQUIRE(x1 && x2 && y && params, "%s: sample arrays and params must not be null", who);
+    XAD_REQUIRE(total > 0 && batch > 0 && epochs >= 0, "%s: total, batch must be positive and epochs non-negative", who);
+    XAD_REQUIRE(lr_first > 0.0 && lr_last > 0.0, "%s: learning rates must be positive", who);
+    XAD_REQUIRE(epochs <= XAD_LINREG_STATIC_MAX_EPOCHS,
+                "%s: %d steps exceed the %d steps one call may queue; split the run into several calls", who, epochs,
+                XAD_LINREG_STATIC_MAX_EPOCHS);
+    double* sums = nullptr;
+    if (int st = scratch_of_current_device(&sums)) return st;
+    return queue_sgd(xad::as_stream(stream), sums, total, x1, x2, y, params, batch, epochs, lr_first, lr_last, seed,
+                     loss_history);
 }
 
 extern "C" int xad_host_linreg_gradient_f64(size_t n, size_t total, const double* x1, const double* x2,

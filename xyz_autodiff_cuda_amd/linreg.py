@@ -57,10 +57,14 @@ def batch_gradient(x1, x2, y, params, rows=None, strategy=WAVE_LDS, out=None, st
     return out
 
 
-def sgd(x1, x2, y, params, batch, epochs, lr_first=1e-4, lr_last=1e-6, seed=0, want_history=False, stream=None):
+def sgd(x1, x2, y, params, batch, epochs, lr_first=1e-4, lr_last=1e-6, seed=0, want_history=False, stream=None,
+        history=None, static_scratch=False):
     """Runs `epochs` steps on the device, updating `params` in place; returns the loss history or None.
 
     Defaults are the reference's learning rates (linear_regression_sgd.cu:26-27).
+    static_scratch=True calls xad_linreg_sgd_f64_static: no device allocation inside the call (pass
+    `history`, a float64 CUDA tensor of `epochs` elements, to keep this wrapper from allocating one
+    too), and the call only queues the work: synchronise the stream before reading the results.
     """
     import torch
 
@@ -68,13 +72,18 @@ def sgd(x1, x2, y, params, batch, epochs, lr_first=1e-4, lr_last=1e-6, seed=0, w
     _check_samples(x1, x2, y)
     if not (params.is_cuda and params.dtype == torch.float64 and params.is_contiguous() and params.numel() == 4):
         raise ValueError("params must be a contiguous float64 CUDA tensor of 4 elements")
-    history = torch.empty(epochs, dtype=torch.float64, device=x1.device) if want_history else None
+    if history is not None:
+        if not (history.is_cuda and history.dtype == torch.float64 and history.is_contiguous() and history.numel() >= epochs):
+            raise ValueError("history must be a contiguous float64 CUDA tensor of at least `epochs` elements")
+    elif want_history:
+        history = torch.empty(epochs, dtype=torch.float64, device=x1.device)
     s = stream if stream is not None else torch.cuda.current_stream(x1.device)
+    name = "xad_linreg_sgd_f64_static" if static_scratch else "xad_linreg_sgd_f64"
     with torch.cuda.device(x1.device):
-        st = lib.xad_linreg_sgd_f64(x1.numel(), x1.data_ptr(), x2.data_ptr(), y.data_ptr(), params.data_ptr(),
-                                    int(batch), int(epochs), float(lr_first), float(lr_last), int(seed),
-                                    history.data_ptr() if history is not None else None, s.cuda_stream)
-    _lib.check(st, "xad_linreg_sgd_f64")
+        st = getattr(lib, name)(x1.numel(), x1.data_ptr(), x2.data_ptr(), y.data_ptr(), params.data_ptr(),
+                                int(batch), int(epochs), float(lr_first), float(lr_last), int(seed),
+                                history.data_ptr() if history is not None else None, s.cuda_stream)
+    _lib.check(st, name)
     return history
 
 
