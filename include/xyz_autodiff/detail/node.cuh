@@ -16,6 +16,18 @@
 //             operand's own backward.  Nodes fire in reverse topological
 //             order, each exactly once, with their gradient complete.
 //
+// Several roots may share a sub-graph: forward each root, seed each, backward
+// each; the shared nodes fire when the last root has released them, as with the
+// counts of xyz-autodiff-cuda (operation.cuh:53-83).  A shared node keeps the
+// value of its first evaluation until it has fired, so operands must not change
+// between the forward passes of two such roots.
+//
+// A forward() that no backward() follows leaves visits registered.  Every node
+// remembers whether it has registered visits that were never released, and the
+// next forward() of that node first withdraws exactly those (recursively, through
+// operands whose count drops to zero), so forward(); forward(); backward() works
+// and never disturbs the visits of another root.
+//
 // All counts are compile-time constants once the graph is inlined, so none of
 // this survives into the ISA: it only decides which calls are emitted.
 //
@@ -39,14 +51,19 @@ namespace detail {
 template <typename X>
 concept HasVisitProtocol = requires(X x) {
     x.xad_visit();
-    x.xad_reset();
+    x.xad_unvisit();
 };
 
-// Forget the consumer counts left behind by an earlier pass that was never
-// followed by a backward.
+// Takes back one visit that will never be released (its consumer is about to
+// be evaluated again).  A node of the three-call protocol can only be told
+// that one consumer is gone.
 template <typename X>
-XAD_INLINE void reset_operand(X& x) {
-    if constexpr (HasVisitProtocol<X>) x.xad_reset();
+XAD_INLINE void unvisit_operand(X& x) {
+    if constexpr (HasVisitProtocol<X>) {
+        x.xad_unvisit();
+    } else if constexpr (OperationNode<X>) {
+        (void)x.decrement_ref_count_and_check();
+    }
 }
 
 template <typename X>
@@ -127,16 +144,17 @@ public:
 
     // A moved node starts with no registered consumers.
     XAD_HD Node(Node&& other) noexcept
-        : logic_(other.logic_), in_(other.in_), out_(other.out_), pending_(0) {}
+        : logic_(other.logic_), in_(other.in_), out_(other.out_), pending_(0), owes_release_(false) {}
 
     // Construction records the operands; nothing is evaluated until forward().
-    XAD_HD Node(const Logic& logic, Ins&... ins) : logic_(logic), in_{ins...}, out_(), pending_(0) {}
+    XAD_HD Node(const Logic& logic, Ins&... ins)
+        : logic_(logic), in_{ins...}, out_(), pending_(0), owes_release_(false) {}
 
     // ---- evaluation -------------------------------------------------------
 
     // Evaluates the whole sub-graph below this node, each node once.
     XAD_INLINE void forward() {
-        in_.each([](auto& x) { reset_operand(x); });
+        withdraw();
         evaluate();
     }
 
@@ -145,6 +163,7 @@ public:
     XAD_INLINE void backward() {
         const output_type& out = out_;
         in_.all([&](auto&... xs) { logic_.backward(out, xs...); });
+        owes_release_ = false;
         in_.each([](auto& x) { release_operand(x); });
     }
 
@@ -155,6 +174,7 @@ public:
     // is passed twice to one node is perturbed (and credited) once per slot.
     XAD_INLINE void backward_numerical(const value_type delta = value_type(1e-5)) {
         in_.each([&](auto& x) { this->perturb(x, delta); });
+        owes_release_ = false;
         in_.each([&](auto& x) { release_operand_numerical(x, delta); });
     }
 
@@ -174,14 +194,14 @@ public:
     // ---- consumer bookkeeping --------------------------------------------
 
     XAD_INLINE void increment_ref_count() { ++pending_; }
-    XAD_INLINE bool decrement_ref_count_and_check() { return --pending_ == 0; }
+    // A release without a matching visit is ignored rather than wrapping the count.
+    XAD_INLINE bool decrement_ref_count_and_check() { return pending_ != 0 && --pending_ == 0; }
 
     XAD_INLINE void xad_visit() {
         if (pending_++ == 0) evaluate();
     }
-    XAD_INLINE void xad_reset() {
-        pending_ = 0;
-        in_.each([](auto& x) { reset_operand(x); });
+    XAD_INLINE void xad_unvisit() {
+        if (pending_ != 0 && --pending_ == 0) withdraw();
     }
 
     // ---- the node as a differentiable variable ---------------------------
@@ -205,8 +225,17 @@ private:
     // with every evaluation, so a graph object can be run any number of times.
     XAD_INLINE void evaluate() {
         in_.each([](auto& x) { visit_operand(x); });
+        owes_release_ = true;
         out_.zero_grad();
         in_.all([&](const auto&... xs) { logic_.forward(out_, xs...); });
+    }
+
+    // Takes back the visits of an evaluation of this node that no backward followed.
+    XAD_INLINE void withdraw() {
+        if (owes_release_) {
+            owes_release_ = false;
+            in_.each([](auto& x) { unvisit_operand(x); });
+        }
     }
 
     XAD_INLINE void seed() {
@@ -238,6 +267,7 @@ private:
     Operands<Ins...> in_;
     output_type out_;
     std::uint8_t pending_;
+    bool owes_release_;  // visits registered with the operands and not yet released
 };
 
 }  // namespace detail

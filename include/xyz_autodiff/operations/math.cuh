@@ -53,8 +53,10 @@ XAD_INLINE float exp(float x) {
     e = ::fmaf(x, kLog2eLo, e);
     const float r = exp2_raw(t);
     const float refined = ::fmaf(r, e * kLn2, r);
-    // r == inf would turn the refinement into inf * 0 or inf - inf.
-    return r == std::numeric_limits<float>::infinity() ? r : refined;
+    // At both ends of the range r is already the answer and the refinement is not: r == inf turns it
+    // into inf * 0 or inf - inf, and for x = -inf or a product that overflowed to -inf (r == 0) the
+    // lost part e is itself inf or NaN.
+    return (r == std::numeric_limits<float>::infinity() || r == 0.0f) ? r : refined;
 }
 
 // sin and cos of one argument from a single reduction.

@@ -82,6 +82,14 @@ def parallel_accumulation(threads, block):
     return out
 
 
+def managed_accumulation(threads):
+    """Gradient sums of `threads` add_grad calls on hipMallocManaged memory: (float: 2 sums, double: 2 sums)."""
+    out = np.zeros(4, np.float64)
+    rc = load().xad_test_managed_accumulation(ctypes.c_size_t(threads), out.ctypes.data_as(ctypes.c_void_p))
+    assert rc == 0
+    return out
+
+
 def shared_accumulation(blocks, threads):
     out = np.zeros(2 * blocks, np.float64)
     rc = load().xad_test_shared_accumulation(ctypes.c_int(blocks), ctypes.c_int(threads), out.ctypes.data_as(ctypes.c_void_p))

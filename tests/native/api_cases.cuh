@@ -67,6 +67,25 @@ private:
     unsigned char count_ = 0;
 };
 
+// A user-written three-operand logic: y = a * b + c, element-wise (the contract of
+// TernaryLogicConcept, include/xyz_autodiff/concept/core_logic.cuh:44-54 of the reference).
+template <std::size_t Dim>
+struct UserMulAddLogic {
+    static constexpr std::size_t outputDim = Dim;
+    template <typename Output, typename A, typename B, typename C>
+    XAD_HD void forward(Output& out, const A& a, const B& b, const C& c) const {
+        for (std::size_t i = 0; i < Dim; ++i) out[i] = a[i] * b[i] + c[i];
+    }
+    template <typename Output, typename A, typename B, typename C>
+    XAD_HD void backward(const Output& out, A& a, B& b, C& c) const {
+        for (std::size_t i = 0; i < Dim; ++i) {
+            a.add_grad(i, out.grad(i) * b[i]);
+            b.add_grad(i, out.grad(i) * a[i]);
+            c.add_grad(i, out.grad(i));
+        }
+    }
+};
+
 XAD_HD inline int run_case(int id, double* out) {
     int n = 0;
     auto put = [&](double v) { out[n++] = v; };
@@ -413,6 +432,83 @@ XAD_HD inline int run_case(int id, double* out) {
                     if (!numerical) put(loss[0]);
                     for (int j = 0; j < 4; ++j) put(diff[j]);
                 }
+            }
+            break;
+        }
+        case 16: {  // TernaryOperation (operation.cuh:382-623 of the reference) with a user logic, y = a b + c
+            using V2 = Variable<2, double>;
+            UserMulAddLogic<2> fma_logic;
+            {   // three leaves: values, analytic gradients, then the numerical ones
+                V2 a, b, c;
+                a[0] = 1.5; a[1] = -2.0; b[0] = 0.5; b[1] = 3.0; c[0] = 0.25; c[1] = -1.0;
+                TernaryOperation<2, UserMulAddLogic<2>, V2, V2, V2> y(fma_logic, a, b, c);
+                y.run();
+                put(y[0]); put(y[1]);
+                put(a.grad(0)); put(a.grad(1)); put(b.grad(0)); put(b.grad(1)); put(c.grad(0)); put(c.grad(1));
+                a.zero_grad(); b.zero_grad(); c.zero_grad();
+                y.run_numerical(1e-6);
+                put(a.grad(0)); put(a.grad(1)); put(b.grad(0)); put(b.grad(1)); put(c.grad(0)); put(c.grad(1));
+            }
+            {   // operands that are nodes, one of them in two slots: y = e * e + n, e = exp(x), n = -x
+                //   d y / d x = 2 e^2x - 1
+                Variable<1, double> x(0.3);
+                auto e = op::exp(x);
+                auto n = op::neg(x);
+                UserMulAddLogic<1> fma1;
+                TernaryOperation<1, UserMulAddLogic<1>, decltype(e), decltype(e), decltype(n)> y(fma1, e, e, n);
+                y.run();
+                put(y[0]); put(x.grad(0));
+            }
+            {   // a ternary node consumed twice: z = y + y^2 with y = a b + c (3.5): d z / d y = 1 + 2 y = 8
+                Variable<1, double> a(2.0), b(1.5), c(0.5);
+                UserMulAddLogic<1> fma1;
+                TernaryOperation<1, UserMulAddLogic<1>, Variable<1, double>, Variable<1, double>, Variable<1, double>> y(fma1, a, b, c);
+                auto y2 = op::squared(y);
+                auto z = y + y2;
+                z.run();
+                put(z[0]); put(a.grad(0)); put(b.grad(0)); put(c.grad(0));
+            }
+            break;
+        }
+        case 17: {  // several roots over one shared node, and forward passes that no backward follows
+            {   // s = exp(x); r1 = -s, r2 = s^2; forward both, seed both, backward both:
+                //   d (r1 + r2) / d x = (2 s - 1) s   (the counts of operation.cuh:53-83 of the reference)
+                Variable<1, double> x(0.5);
+                auto s = op::exp(x);
+                auto r1 = op::neg(s);
+                auto r2 = op::squared(s);
+                r1.forward();
+                r2.forward();
+                r1.add_grad(0, 1.0);
+                r2.add_grad(0, 1.0);
+                r1.backward();
+                put(x.grad(0));  // s has one more consumer to hear from: nothing has reached x yet
+                r2.backward();
+                put(r1[0]); put(r2[0]); put(x.grad(0));
+            }
+            {   // forward twice, then backward: the first pass leaves nothing behind
+                Variable<1, double> x(0.5);
+                auto s = op::exp(x);
+                auto r = op::squared(s);
+                r.forward();
+                x[0] = 0.25;  // and the second pass sees the new value
+                r.forward();
+                r.add_grad(0, 1.0);
+                r.backward();
+                put(r[0]); put(x.grad(0));  // e^0.5, 2 e^0.5
+            }
+            {   // a root forwarded and abandoned does not disturb another root over the same node
+                Variable<1, double> x(0.5);
+                auto s = op::exp(x);
+                auto abandoned = op::neg(s);
+                auto r = op::squared(s);
+                abandoned.forward();
+                abandoned.forward();  // takes back its own visit first: s still has exactly one
+                r.run();
+                put(x.grad(0));  // s waits for `abandoned`: nothing yet
+                abandoned.add_grad(0, 1.0);
+                abandoned.backward();
+                put(x.grad(0));  // (2 s - 1) s
             }
             break;
         }

@@ -9,6 +9,7 @@
 #include <cstring>
 
 #include "api_cases.cuh"
+#include <xyz_autodiff/util/hip_managed_ptr.cuh>
 #include "tester_suite.cuh"
 #include "concept_checks.cuh"
 
@@ -150,7 +151,35 @@ __global__ void shared_accumulation_kernel(double* per_block) {
     }
 }
 
+// VariableRef::add_grad from every thread on memory that the host can also reach (hipMallocManaged): the
+// pairing the tests of xyz-autodiff-cuda use throughout (cuda_managed_ptr + VariableRef, e.g.
+// tests/test_parallel_gradient_accumulation.cu:60-99).
+template <typename T>
+__global__ void managed_accumulation_kernel(T* values, T* grads, std::size_t threads) {
+    const std::size_t tid = static_cast<std::size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (tid >= threads) return;
+    VariableRef<2, T> v(values, grads);
+    v.add_grad(0, T(1));
+    v.add_grad(1, T(0.5) * v[1]);
+}
+
 bool ok(hipError_t e) { return e == hipSuccess; }
+
+template <typename T>
+int managed_accumulation(std::size_t threads, double* out2) {
+    auto values = makeHipManagedArray<T>(2);
+    auto grads = makeHipManagedArray<T>(2);
+    if (!values || !grads) return -2;
+    values[0] = T(0);
+    values[1] = T(4);  // written by the host, read by the device
+    grads[0] = grads[1] = T(0);
+    hipLaunchKernelGGL(managed_accumulation_kernel<T>, dim3(static_cast<unsigned>((threads + 255) / 256)), dim3(256), 0, 0,
+                       values.get(), grads.get(), threads);
+    if (!ok(hipGetLastError()) || !ok(hipDeviceSynchronize())) return -2;
+    out2[0] = static_cast<double>(grads[0]);  // read by the host after the wait
+    out2[1] = static_cast<double>(grads[1]);
+    return 0;
+}
 
 }  // namespace
 
@@ -215,6 +244,12 @@ extern "C" int xad_test_parallel_accumulation(std::size_t threads, int block, do
     (void)hipFree(d_values);
     (void)hipFree(d_grads);
     return rc;
+}
+
+// out4: the two gradients for float, then for double.
+extern "C" int xad_test_managed_accumulation(std::size_t threads, double* out4) {
+    if (int rc = managed_accumulation<float>(threads, out4)) return rc;
+    return managed_accumulation<double>(threads, out4 + 2);
 }
 
 extern "C" int xad_test_shared_accumulation(int blocks, int threads, double* per_block) {

@@ -30,6 +30,33 @@ template <std::size_t Out, typename Logic, typename A, typename B>
 inline constexpr bool binary_ok = is_node<BinaryOperation<Out, Logic, A, B>> && BinaryOperation<Out, Logic, A, B>::size == Out &&
                                   Logic::outputDim == Out;
 
+template <std::size_t Out, typename Logic, typename A, typename B, typename C>
+inline constexpr bool ternary_ok = is_node<TernaryOperation<Out, Logic, A, B, C>> &&
+                                   TernaryOperation<Out, Logic, A, B, C>::size == Out && Logic::outputDim == Out;
+
+// The library ships no three-operand logic; the contract of TernaryLogicConcept / TernaryOperation
+// (concept/core_logic.cuh:44-54 and operations/operation.cuh:382-623 of the reference) is asserted with the
+// smallest logic a user could write.
+template <std::size_t Dim>
+struct MulAddLogic {
+    static constexpr std::size_t outputDim = Dim;
+    template <typename Output, typename A, typename B, typename C>
+    XAD_HD void forward(Output& out, const A& a, const B& b, const C& c) const {
+        for (std::size_t i = 0; i < Dim; ++i) out[i] = a[i] * b[i] + c[i];
+    }
+    template <typename Output, typename A, typename B, typename C>
+    XAD_HD void backward(const Output& out, A& a, B& b, C& c) const {
+        for (std::size_t i = 0; i < Dim; ++i) {
+            a.add_grad(i, out.grad(i) * b[i]);
+            b.add_grad(i, out.grad(i) * a[i]);
+            c.add_grad(i, out.grad(i));
+        }
+    }
+};
+struct NotALogic {
+    static constexpr std::size_t outputDim = 2;
+};
+
 // Every logic over leaves of one kind (Variable or VariableRef) and one value type.
 template <template <std::size_t, typename> class Leaf, typename T>
 constexpr bool all_logics() {
@@ -57,6 +84,12 @@ constexpr bool all_logics() {
     static_assert(binary_ok<3, op::MulLogic<L3, L3>, L3, L3> && binary_ok<3, op::DivLogic<L3, L3>, L3, L3>);
     static_assert(binary_ok<4, op::MatMulLogic<2, 2, 2, L4, L4>, L4, L4> && binary_ok<9, op::MatMulLogic<3, 3, 3, L9, L9>, L9, L9>);
     static_assert(binary_ok<2, op::MatMulLogic<2, 3, 1, L6, L3>, L6, L3> && binary_ok<2, op::MatMulLogic<1, 3, 2, L3, L6>, L3, L6>);
+    // three operands: leaves, and nodes of the other arities as operands
+    static_assert(TernaryLogicConcept<MulAddLogic<2>, L2, L2, L2, Variable<2, T>> && ternary_ok<2, MulAddLogic<2>, L2, L2, L2>);
+    static_assert(TernaryLogicParameterConcept<L2, L2, L2>);
+    static_assert(!TernaryLogicConcept<NotALogic, L2, L2, L2, Variable<2, T>> && !TernaryLogicConcept<op::AddLogic<L2, L2>, L2, L2, L2, Variable<2, T>>);
+    static_assert(ternary_ok<2, MulAddLogic<2>, UnaryOperation<2, op::ExpLogic<2>, L2>, L2, BinaryOperation<2, op::MulLogic<L2, L2>, L2, L2>>);
+    static_assert(unary_ok<2, op::NegLogic<2>, TernaryOperation<2, MulAddLogic<2>, L2, L2, L2>>);
     // splatting logics
     static_assert(binary_ok<4, op::CovarianceMatrixGenerationLogic<L2, L1>, L2, L1> && unary_ok<3, op::MatrixToCovariance3ParamLogic<L4>, L4>);
     static_assert(binary_ok<3, op::ScaleRotationToCovariance3ParamLogic<L2, L1>, L2, L1>);

@@ -27,6 +27,11 @@ EXPECTED = {
     10: [6, 4] + [9, 4] + [12, 7] + [-1.2, 2, 2] + [12, 8, 6, 16],
     11: [2.5, 1.5, 0.75, 1.125, 1.5, 0.75, 1.125],
     12: [4.625, 2.5, -3.5] + [2 * (E + E ** -2), 2 * E, 2 * E ** -2],
+    # TernaryOperation, y = a b + c: values; d a = b, d b = a, d c = 1 (analytic, then numerical);
+    # node operands: e^0.6 - 0.3, 2 e^0.6 - 1; a ternary node consumed twice: 3.5 + 3.5^2, 8 (b, a, 1)
+    16: [1.0, -7.0] + [0.5, 3.0, 1.5, -2.0, 1.0, 1.0] * 2 + [E ** 0.6 - 0.3, 2 * E ** 0.6 - 1] + [15.75, 12.0, 16.0, 8.0],
+    # roots sharing a node: 0 until the last root has released it, then (2 s - 1) s with s = e^0.5
+    17: [0.0, -E ** 0.5, E, (2 * E ** 0.5 - 1) * E ** 0.5] + [E ** 0.5, 2 * E ** 0.5] + [0.0, (2 * E ** 0.5 - 1) * E ** 0.5],
 }
 
 
@@ -105,3 +110,12 @@ def test_concurrent_add_grad_on_lds(gpu, blocks, threads):
     """tests/test_shared_memory_atomic.cu:102-109 and :179-187 of the reference."""
     got = _native.shared_accumulation(blocks, threads)
     assert np.all(got[:, 0] == threads) and np.all(got[:, 1] == 2 * threads)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("threads", [1, 64, 10_000, 1 << 20])
+def test_concurrent_add_grad_on_managed_memory(gpu, threads):
+    """VariableRef over makeHipManagedArray memory, the pairing of the reference's tests (cuda_managed_ptr,
+    tests/test_parallel_gradient_accumulation.cu:60-99): no contribution may be lost, in float or double."""
+    got = _native.managed_accumulation(threads)
+    assert list(got) == [threads, 2.0 * threads, threads, 2.0 * threads], got

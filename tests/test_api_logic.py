@@ -67,3 +67,27 @@ def test_fp32_exp_and_sincos_are_accurate_to_two_ulp():
         arg = np.float64(np.float32(np.array([x, -x, x / 3])))
         worst = max(worst, np.abs(s - np.sin(arg)).max(), np.abs(c - np.cos(arg)).max())
     assert worst <= 2.5e-7, worst  # absolute: two ulp of values near one
+
+
+def _special_values(device):
+    inf, big = np.inf, float(np.finfo(np.float32).max)
+    e, _, _ = _native.eval_logic("exp", [np.array([-inf, -big, -104.0])], dtype=np.float32, device=device)
+    assert np.all(e == 0.0), e
+    e, _, _ = _native.eval_logic("exp", [np.array([inf, big, 89.0])], dtype=np.float32, device=device)
+    assert np.all(e == inf), e
+    e, _, _ = _native.eval_logic("exp", [np.array([np.nan, 0.0, -0.0])], dtype=np.float32, device=device)
+    assert np.isnan(e[0]) and e[1] == 1.0 and e[2] == 1.0, e
+    s, _, _ = _native.eval_logic("sigmoid", [np.array([inf, big, 200.0])], dtype=np.float32, device=device)
+    assert np.all(s == 1.0), s
+    s, _, _ = _native.eval_logic("sigmoid", [np.array([-inf, -big, -200.0])], dtype=np.float32, device=device)
+    assert np.all(s == 0.0), s
+
+
+def test_fp32_exp_and_sigmoid_at_the_ends_of_the_range():
+    """expf of the C library gives 0 at -inf and below the range, inf above it; sigmoid follows with 0 and 1."""
+    _special_values(device=False)
+
+
+@pytest.mark.gpu
+def test_fp32_exp_and_sigmoid_at_the_ends_of_the_range_on_gpu(gpu):
+    _special_values(device=True)
