@@ -70,23 +70,6 @@ int xad_chain_forward_backward_f32(size_t n,
                                    float* d_o, float* d_px, float* d_py,
                                    void* stream);
 
-/* Same computation with the lane-to-address mapping chosen by the caller:
- * problems_per_lane = 1 (4-byte accesses, the default mapping of the entry point
- * above) or 4 (16-byte accesses; needs all arrays 16-byte aligned, otherwise, and
- * for the last n % 4 problems, the 4-byte kernel is used).  Results are identical;
- * exists so both mappings can be measured.  No counterpart in the reference. */
-int xad_chain_forward_backward_f32_layout(size_t n,
-                                          const float* sx, const float* sy, const float* theta,
-                                          const float* o, const float* px, const float* py,
-                                          float* w, float* d_sx, float* d_sy, float* d_theta,
-                                          float* d_o, float* d_px, float* d_py,
-                                          int problems_per_lane, void* stream);
-
-/* dst[i] = src[i] for n floats on the device, with the access pattern of the
- * kernel above: a copy of known size to calibrate counters and bandwidth against.
- * No counterpart in the reference. */
-int xad_stream_copy_f32(size_t n, const float* src, float* dst, void* stream);
-
 /* The same graph from the same templates, compiled for the host and run on
  * `num_threads` host threads (<= 0: all hardware threads).  Host pointers.
  * Synchronous.  This is the "host-core run of the per-thread templates"; GPU
@@ -370,38 +353,6 @@ int xad_linreg_sgd_f64_static(size_t total, const double* x1, const double* x2, 
 int xad_host_linreg_gradient_f64(size_t n, size_t total,
                                  const double* x1, const double* x2, const double* y, const int* rows,
                                  const double* params, double* out);
-
-/* ---------------------------------------------------------------------------
- * Hardware probe behind the accumulator's design: shader cycles the LDS pipeline
- * of a CU spends on one wavefront-wide atomic add (16 wavefronts of one block
- * issuing back to back), by element type (0 float, 1 double, 2 uint32, 3 uint64)
- * and address pattern (0 sixty-four distinct addresses, 1 one address, 2 sixteen
- * lanes on one address, 3 eight lanes per address, 4 stride of six elements).
- * Synchronous; allocates and frees small device buffers.  No counterpart in the
- * reference.
- */
-int xad_probe_lds_atomic_cycles(int element, int pattern, double* cycles_per_instruction);
-
-/* Resources of the default kernel of xad_chain_forward_backward_f32 as the loaded
- * code object and the current device report them: vector registers per lane,
- * scratch (spill) bytes per lane, static LDS bytes per block, lanes per block, and
- * how many such blocks one compute unit holds at once.  out[5] in that order.
- * No counterpart in the reference.
- */
-int xad_chain_kernel_resources(int* out);
-
-/* Hardware probe behind the default kernel of xad_chain_forward_backward_f32: the
- * same kernel (one problem per lane, non-temporal loads) with its seven results
- * stored as 0 write-through stores (relaxed atomic stores at agent scope, the
- * library's choice), 1 plain stores, 2 non-temporal stores.  Same arguments and
- * results as xad_chain_forward_backward_f32; only the time differs.  No
- * counterpart in the reference.
- */
-int xad_probe_chain_store_policy(int policy, size_t n,
-                                 const float* sx, const float* sy, const float* theta,
-                                 const float* o, const float* px, const float* py,
-                                 float* w, float* d_sx, float* d_sy, float* d_theta,
-                                 float* d_o, float* d_px, float* d_py, void* stream);
 
 /* ---------------------------------------------------------------------------
  * Synthetic inputs: counter-based generator, element i of a fill is a pure

@@ -23,19 +23,24 @@
 // the 64 addresses are distinct, plus about 3 cycles per lane that shares an
 // address with another.  So partial sums are kept in fp64 (which also makes them
 // more accurate than the fp32 running sums of plain atomics).  Two ways to take
-// the sharing lanes out of the LDS instruction: a small table can be replicated,
-// lane l adding into copy l % replicas (no extra instructions; the fastest at
-// every slot count measured), or level 1 can sum a group of m sharing lanes
+// the sharing lanes out of the LDS instruction: rows can be replicated, lane l
+// adding into copy l % replicas (no extra instructions; the fastest at every
+// slot count measured): every row of a small table, or only the first
+// `hot_rows` rows of a large one, which under a skewed law over the slot index
+// take most of the adds; or level 1 can sum a group of m sharing lanes
 // first, which costs about 60 VALU issue cycles per group and saves about
 // 3 m Width LDS cycles (MinGroup = 4 is where that starts to pay).
 //
 // The LDS table holds `capacity` slots of Width values, stored element-major
 // (all slots' element 0, then element 1, ...) so that the lanes of one
 // instruction, which all address the same element, spread over the banks.  If
-// all num_slots fit, slot s uses row s.  Otherwise rows are claimed on first use through a tag
-// array (hashed, one probe, no eviction): a slot that finds its row taken by
-// another slot falls through to a global atomic.  Under skewed access the hot
-// slots arrive first and most often, so they own the rows.
+// all num_slots fit, slot s uses row s.  Otherwise either the first `capacity`
+// slots own the rows (no tags, no probing: right when the hot slots are the
+// low-numbered ones, as with a Zipf law over the slot index) or rows are
+// claimed on first use through a tag array (hashed, one probe, no eviction:
+// under skewed access the hot slots arrive first and most often, so they own
+// the rows wherever they are).  A slot without a row falls through to global
+// atomics.
 //
 // Collective-call rules: construct(), add(), add_one() and flush() must be
 // reached by every lane of every wavefront of the block, in uniform control
@@ -120,54 +125,73 @@ public:
     static constexpr int kEmpty = -1;
 
     // Bytes of LDS the block must provide for `capacity` rows.
+    // (tagged: rows claimed on first use, which needs a tag per row)
     __host__ __device__ static constexpr std::size_t lds_bytes(int capacity, bool tagged) {
         if (S == Strategy::GlobalAtomics) return 0;
         return static_cast<std::size_t>(capacity) * Width * sizeof(TableT) + (tagged ? static_cast<std::size_t>(capacity) * 4 : 0);
     }
 
-    // `lds`: at least lds_bytes(capacity, num_slots > capacity) bytes, 16-byte aligned.
-    // `capacity` must be a power of two when num_slots > capacity (tagged mode).
+    // `lds`: at least lds_bytes(capacity, tagged) bytes, 16-byte aligned.  `capacity`: rows of the table.
     // `global`: num_slots rows of Width values, already initialised; row s starts at
     // global + s * row_stride (row_stride = Width for a dense row-major array; a larger
     // stride lets several accumulators share one array, each owning every k-th row).
-    // `replicas` (a power of two; 1 = none): a small table is kept that many times and lane l
-    // adds into copy l % replicas, so lanes of one instruction that share a slot no longer
-    // share an address (each sharing lane costs an LDS atomic about 3 cycles); flush() adds the
-    // copies up.  Needs capacity >= replica_rows(num_slots) * replicas.
+    // `claim_rows` (only matters when the slots do not all get a row): true = rows are claimed on
+    // first use through the tag array (capacity must then be a power of two, replicas 1); false = the
+    // first slots own the rows and no tags are kept.
+    // `replicas` (a power of two; 1 = none) and `hot_rows` (negative = every slot): slots below
+    // hot_rows are kept in that many copies and lane l adds into copy l % replicas, so lanes of one
+    // instruction that share such a slot no longer share an address (each sharing lane costs an LDS
+    // atomic about 3 cycles); flush() adds the copies up.  The copies take (replicas - 1) *
+    // (hot_rows | 1) rows of the capacity, after the rows of the slots themselves (rows_for()).
     // Clears the table; ends with a block barrier.
     __device__ BlockAccumulator(void* lds, int capacity, T* global, int num_slots, int row_stride = Width,
-                                int replicas = 1)
+                                int replicas = 1, bool claim_rows = true, int hot_rows = -1)
         : table_(static_cast<TableT*>(lds)),
           tags_(reinterpret_cast<int*>(static_cast<TableT*>(lds) + static_cast<std::size_t>(capacity) * Width)),
           global_(global),
           capacity_(capacity),
           num_slots_(num_slots),
           row_stride_(row_stride),
-          tagged_(replicas == 1 && num_slots > capacity),
+          tagged_(replicas == 1 && num_slots > capacity && claim_rows),
           shift_(32 - __builtin_ctz(static_cast<unsigned>(capacity))),
-          replicas_(replicas),
-          my_copy_(static_cast<int>(wave::lane_id() & static_cast<unsigned>(replicas - 1)) * replica_rows(num_slots)) {
+          replicas_(replicas) {
+        hot_ = replicas > 1 ? (hot_rows < 0 || hot_rows > num_slots ? num_slots : hot_rows) : 0;
+        hot_stride_ = hot_ | 1;
+        // rows left for the slots themselves once the copies of the hot ones are set aside
+        // (the copies start at an odd row: main_rows_ | 1 must fit in front of them)
+        const int in_front = capacity - (replicas - 1) * hot_stride_;
+        const int left = replicas > 1 ? ((in_front & 1) ? in_front : in_front - 1) : capacity;
+        main_rows_ = tagged_ ? capacity : (num_slots < left ? num_slots : left);
+        if (hot_ > main_rows_) hot_ = main_rows_;
+        copies_base_ = main_rows_ | 1;
+        const int copy = static_cast<int>(wave::lane_id() & static_cast<unsigned>(replicas - 1));
+        my_copy_ = copy == 0 ? 0 : copies_base_ + (copy - 1) * hot_stride_;
         clear();
     }
 
-    // Rows one copy of a replicated table occupies: odd, so that the copies of a slot fall
-    // into different LDS banks.
-    __host__ __device__ static constexpr int replica_rows(int num_slots) { return num_slots | 1; }
+    // Rows a table needs for `slots` slots of which the first `hot_rows` are kept in `replicas` copies.
+    __host__ __device__ static constexpr int rows_for(int slots, int replicas, int hot_rows) {
+        return replicas > 1 ? (slots | 1) + (replicas - 1) * (hot_rows | 1) : slots;
+    }
+
+    // Rows a wavefront can stage per round of the spill path below.
+    static constexpr int kStageRows = 16;
 
     // Bytes of LDS for use_spill_staging() in a block of `threads` lanes.
     __host__ __device__ static constexpr std::size_t spill_bytes(int threads) {
-        return static_cast<std::size_t>(threads) * (Width + 1) * 4;
+        return static_cast<std::size_t>(threads / 64) * kStageRows * (Width + 1) * 4;
     }
 
-    // With Spill (tagged tables of 4-byte values): contributions that find no row are not sent
-    // to `global` lane by lane (Width instructions, each touching up to 64 rows) but are first
-    // gathered per wavefront in `staging` (spill_bytes(blockDim.x) bytes of LDS, 4-byte aligned)
-    // and written out with consecutive lanes on consecutive elements of consecutive rows, which
-    // cuts the number of memory requests several times.  Must be called before the first add();
-    // add() must then be reached by all lanes of a wavefront together whatever the strategy.
+    // With Spill (tables of 4-byte values that do not hold every slot): contributions that find no
+    // row are not sent to `global` lane by lane (Width instructions, each touching up to 64 rows) but
+    // are first gathered per wavefront in `staging` (spill_bytes(blockDim.x) bytes of LDS, 4-byte
+    // aligned), kStageRows at a time, and written out with consecutive lanes on consecutive elements
+    // of consecutive rows, which cuts the number of memory requests several times.  Must be called
+    // before the first add(); add() must then be reached by all lanes of a wavefront together
+    // whatever the strategy.
     __device__ void use_spill_staging(void* staging) {
         static_assert(Spill, "declare the accumulator with Spill = true");
-        spill_ = static_cast<std::uint32_t*>(staging) + (threadIdx.x / 64) * 64 * (Width + 1);
+        spill_ = static_cast<std::uint32_t*>(staging) + (threadIdx.x / 64) * kStageRows * (Width + 1);
     }
 
     // Adds g[0..Width) to slot `slot` (no-op for slot < 0).
@@ -207,13 +231,13 @@ public:
         __syncthreads();
         // e runs over the global layout (slot-major) so the atomics of a
         // wavefront touch consecutive addresses.
-        const int rows = tagged_ ? capacity_ : num_slots_;
-        const int copy_rows = replica_rows(num_slots_);
-        for (int e = threadIdx.x; e < rows * Width; e += blockDim.x) {
+        for (int e = threadIdx.x; e < main_rows_ * Width; e += blockDim.x) {
             const int row = e / Width, element = e % Width;
             const int slot = tagged_ ? tags_[row] : row;
             TableT sum = table_[element * capacity_ + row];
-            for (int copy = 1; copy < replicas_; ++copy) sum += table_[element * capacity_ + copy * copy_rows + row];
+            if (row < hot_)
+                for (int copy = 1; copy < replicas_; ++copy)
+                    sum += table_[element * capacity_ + copies_base_ + (copy - 1) * hot_stride_ + row];
             const T v = static_cast<T>(sum);
             if (slot != kEmpty && v != T(0)) detail::atomic_add(global_ + static_cast<std::size_t>(slot) * row_stride_ + element, v);
         }
@@ -232,7 +256,7 @@ private:
 
     // Row of the LDS table that holds `slot`, or -1 if the slot has none.
     __device__ __forceinline__ int find_row(int slot) {
-        if (!tagged_) return slot + my_copy_;
+        if (!tagged_) return slot < hot_ ? slot + my_copy_ : (slot < main_rows_ ? slot : -1);
         const int row = static_cast<int>((static_cast<unsigned>(slot) * 2654435761u) >> shift_);
         int owner = tags_[row];
         if (owner == kEmpty) {
@@ -262,27 +286,30 @@ private:
 #pragma unroll
             for (int k = 0; k < Width; ++k) detail::atomic_add(table_ + k * capacity_ + row, static_cast<TableT>(g[k]));
         }
-        const bool miss = slot >= 0 && row < 0;
-        const std::uint64_t missing = wave::ballot(miss);
-        if (missing == 0) return;
-        if (miss) {
+        bool miss = slot >= 0 && row < 0;
+        for (std::uint64_t missing = wave::ballot(miss); missing != 0; missing = wave::ballot(miss)) {
+            // this round: the first kStageRows lanes that still have a contribution without a row
             const unsigned before = __builtin_amdgcn_mbcnt_hi(static_cast<unsigned>(missing >> 32),
                                                               __builtin_amdgcn_mbcnt_lo(static_cast<unsigned>(missing), 0u));
-            std::uint32_t* mine = spill_ + before * (Width + 1);
-            mine[0] = static_cast<std::uint32_t>(slot);
+            if (miss && before < static_cast<unsigned>(kStageRows)) {
+                std::uint32_t* mine = spill_ + before * (Width + 1);
+                mine[0] = static_cast<std::uint32_t>(slot);
 #pragma unroll
-            for (int k = 0; k < Width; ++k) mine[1 + k] = __builtin_bit_cast(std::uint32_t, g[k]);
+                for (int k = 0; k < Width; ++k) mine[1 + k] = __builtin_bit_cast(std::uint32_t, g[k]);
+                miss = false;
+            }
+            __builtin_amdgcn_wave_barrier();
+            const int waiting = __builtin_popcountll(missing);
+            const int elements = (waiting < kStageRows ? waiting : kStageRows) * Width;
+            for (int e = static_cast<int>(wave::lane_id()); e < elements; e += 64) {
+                const int entry = e / Width, k = e - entry * Width;
+                const std::uint32_t* staged = spill_ + entry * (Width + 1);
+                const T value = __builtin_bit_cast(T, staged[1 + k]);
+                if (value != T(0))
+                    detail::atomic_add(global_ + static_cast<std::size_t>(staged[0]) * row_stride_ + k, value);
+            }
+            __builtin_amdgcn_wave_barrier();
         }
-        __builtin_amdgcn_wave_barrier();
-        const int elements = __builtin_popcountll(missing) * Width;
-        for (int e = static_cast<int>(wave::lane_id()); e < elements; e += 64) {
-            const int entry = e / Width, k = e - entry * Width;
-            const std::uint32_t* staged = spill_ + entry * (Width + 1);
-            const T value = __builtin_bit_cast(T, staged[1 + k]);
-            if (value != T(0))
-                detail::atomic_add(global_ + static_cast<std::size_t>(staged[0]) * row_stride_ + k, value);
-        }
-        __builtin_amdgcn_wave_barrier();
     }
 
     // Level 1.  Take the slot of the first lane that is still waiting and find
@@ -317,10 +344,14 @@ private:
     int capacity_;
     int num_slots_;
     int row_stride_;
-    bool tagged_;
+    bool tagged_;  // rows claimed on first use (tags_ says by which slot)
     int shift_;
     int replicas_;
-    int my_copy_;  // first row of this lane's copy of the table
+    int main_rows_;    // slots 0 .. main_rows_-1 own rows 0 .. main_rows_-1 (tagged: all rows, claimed)
+    int hot_;          // slots below this are kept in replicas_ copies
+    int hot_stride_;   // rows between two copies (odd, so copies of a slot fall into different banks)
+    int copies_base_;  // first row of the second copy
+    int my_copy_;      // offset of this lane's copy of a hot row (0 for the first copy)
     std::uint32_t* spill_ = nullptr;
 };
 

@@ -94,9 +94,15 @@ class Oracle:
 
     # ---- splatting -----------------------------------------------------------
 
-    def splat_step(self, width, height, params, depth, target, dtype=np.float32, want_grads=True):
+    def splat_step(self, width, height, params, depth, target, dtype=np.float32, want_grads=True, rects_in=None,
+                   want_bounds=False):
         """Tile-binned step on the CPU.  params (9, G).  Returns dict with image (H, W, 3),
-        grads (9, G) or None, loss, pairs, longest_list, seconds (5 stages)."""
+        grads (9, G) or None, loss, pairs, longest_list, seconds (5 stages), rects (G, 4: first/last tile
+        column and row of every Gaussian).  rects_in: bin with these rectangles instead of deriving them
+        (an fp64 run then bins exactly like the fp32 run they came from).  want_bounds adds grad_mass and
+        grad_bound (9, G, float64): the sum of the magnitudes of the per-pixel terms behind every gradient,
+        and a first-order bound on the distance of an fp32 evaluation of the step from this one, and
+        image_bound (H, W, 3), the same kind of bound for the image."""
         dtype = np.dtype(dtype)
         params = np.ascontiguousarray(params, dtype=dtype)
         depth = np.ascontiguousarray(depth, dtype=dtype)
@@ -104,14 +110,24 @@ class Oracle:
         G = params.shape[1]
         image = np.zeros((height, width, 3), dtype)
         grads = np.zeros((9, G), dtype) if want_grads else None
+        rects = np.zeros((G, 4), np.int32)
+        if rects_in is not None:
+            rects_in = np.ascontiguousarray(rects_in, dtype=np.int32)
+            assert rects_in.shape == (G, 4)
+        mass = np.zeros((9, G), np.float64) if want_bounds else None
+        bound = np.zeros((9, G), np.float64) if want_bounds else None
+        image_bound = np.zeros((height, width, 3), np.float64) if want_bounds else None
+        assert want_grads or not want_bounds
         stats = (ctypes.c_long * 2)()
         seconds = (ctypes.c_double * 5)()
-        fn = getattr(self.lib, "oracle_splat_step" + _SUF[dtype])
+        fn = getattr(self.lib, "oracle_splat_step_ex" + _SUF[dtype])
         fn.restype = ctypes.c_double
         P = ctypes.c_void_p
-        loss = fn(ctypes.c_int(width), ctypes.c_int(height), ctypes.c_int(G), params.ctypes.data_as(P), depth.ctypes.data_as(P),
-                  target.ctypes.data_as(P), image.ctypes.data_as(P), grads.ctypes.data_as(P) if want_grads else P(0), stats, seconds)
-        return {"image": image, "grads": grads, "loss": loss, "pairs": stats[0], "longest_list": stats[1], "seconds": list(seconds)}
+        ptr = lambda a: a.ctypes.data_as(P) if a is not None else P(0)
+        loss = fn(ctypes.c_int(width), ctypes.c_int(height), ctypes.c_int(G), ptr(params), ptr(depth), ptr(target), ptr(image),
+                  ptr(grads), stats, seconds, ptr(rects_in), ptr(rects), ptr(mass), ptr(bound), ptr(image_bound))
+        return {"image": image, "grads": grads, "loss": loss, "pairs": stats[0], "longest_list": stats[1], "seconds": list(seconds),
+                "rects": rects, "grad_mass": mass, "grad_bound": bound, "image_bound": image_bound}
 
     def splat_bruteforce(self, width, height, params, depth, target, dtype=np.float64):
         """Every pixel against every Gaussian.  Returns (image, loss)."""

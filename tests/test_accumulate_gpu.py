@@ -132,8 +132,8 @@ def test_rejects_bad_arguments(gpu, xad):
 def test_lds_fp64_atomics_are_the_fast_ones(gpu, xad):
     """The measurement the fp64 LDS table rests on: a wavefront-wide ds_add_f64 to
     distinct addresses must be several times cheaper than a ds_add_f32."""
-    from xyz_autodiff_cuda_amd import accumulate
+    import instruments
 
-    cycles = accumulate.lds_atomic_cycles()
+    cycles = instruments.lds_atomic_cycles()
     assert cycles["f64"]["64_distinct"] * 4 < cycles["f32"]["64_distinct"]
     assert cycles["f64"]["one_address"] > cycles["f64"]["64_distinct"]

@@ -15,8 +15,11 @@ pytestmark = pytest.mark.gpu
 
 
 def _run_gpu(inputs, gpu, offset=0, problems_per_lane=None):
+    """problems_per_lane None: the library (one problem per lane); 1 or 4: the same kernel body with the
+    lane-to-address mapping chosen, from the measurement library (instruments/)."""
     import torch
 
+    import instruments
     from xyz_autodiff_cuda_amd import chain
 
     n = inputs[0].size
@@ -27,7 +30,10 @@ def _run_gpu(inputs, gpu, offset=0, problems_per_lane=None):
         view.copy_(torch.from_numpy(np.ascontiguousarray(a)))
         dev.append(view)
     outs = [torch.full((n + offset,), float("nan"), dtype=torch.float32, device=gpu)[offset:] for _ in range(7)]
-    chain.forward_backward(dev, outs, problems_per_lane=problems_per_lane)
+    if problems_per_lane is None:
+        chain.forward_backward(dev, outs)
+    else:
+        instruments.chain_with_layout(dev, outs, problems_per_lane)
     torch.cuda.synchronize()
     return np.stack([o.cpu().numpy() for o in outs])
 
@@ -71,21 +77,26 @@ def test_both_lane_mappings_and_unaligned_buffers_agree_bitwise(gpu, oracle):
     assert np.array_equal(a, c)
 
 
-def test_store_policies_of_the_probe_agree_bitwise(gpu, xad):
-    """xad_probe_chain_store_policy changes how results are stored, never what is stored."""
+def test_store_policies_of_the_instrument_agree_bitwise(gpu, xad):
+    """The store-policy instrument changes how results are stored, never what is stored."""
     import torch
 
+    import instruments
     from xyz_autodiff_cuda_amd import chain
 
     n = 70_001
     ins = [torch.from_numpy(a).to(gpu) for a in chain_inputs(n, seed=12)]
     want = torch.stack(chain.forward_backward(ins))
-    for policy in chain.STORE_POLICIES:
+    for policy in instruments.STORE_POLICIES:
         outs = [torch.full((n,), float("nan"), dtype=torch.float32, device=gpu) for _ in range(7)]
-        chain.store_policy_probe(ins, outs, policy)
+        instruments.chain_with_store_policy(ins, outs, policy)
         assert torch.equal(torch.stack(outs), want), policy
-    with pytest.raises(xad.XadError, match="policy"):
-        chain.store_policy_probe(ins, outs, 7)
+    with pytest.raises(instruments.InstrumentError, match="policy"):
+        instruments.chain_with_store_policy(ins, outs, 7)
+    copy = instruments.stream_copy(ins[0], torch.zeros_like(ins[0]))
+    assert torch.equal(copy, ins[0])
+    resources = instruments.chain_kernel_resources()
+    assert resources["scratch_bytes"] == 0 and 0 < resources["vgprs"] <= 64 and resources["wavefronts_per_simd"] == 8
 
 
 def test_device_matches_host_build_of_the_same_templates(gpu, xad):

@@ -1,0 +1,182 @@
+"""GPU parity at the benchmark's full sizes, every problem against the CPU oracle, through the C ABI.
+
+  chain          64 Mi problems (6 inputs, value + 6 gradients each), all of them against the fp32 and
+                 the fp64 oracle, in pieces of 8 Mi;
+  accumulation   16 Mi threads, device-drawn Zipf(1.1) slots, 64 / 4096 / 262 144 slots;
+  splatting      exactly 10 000 Gaussians at 512 x 512 and exactly 200 000 at 2048 x 2048 with the
+                 benchmark's scene and target recipe.
+
+Tolerances are the ones of the small-size tests (tests/test_chain_gpu.py, test_accumulate_gpu.py) and, for
+the splatting gradients, a bound that holds for every Gaussian on its merits:
+
+    |gpu - fp64| <= 1e-4 * mass + bound
+
+with mass = the sum of the magnitudes of the per-pixel terms behind that gradient (the scale of the
+rounding of any summation order) and bound = the oracle's first-order bound on the distance of an
+fp32 evaluation of the same step from the fp64 one (ill-conditioned inverse covariances, their effect
+on transmittance and on the colours behind, stop and clamp decisions that rounding can flip; see
+oracle/oracle_splat.inc).  tests/test_oracle_splat.py checks that the fp32 oracle itself stays within
+that bound and that a 1 % error does not.
+
+Every test also reports (in its output and in its assertion messages) which fraction of the problems
+meets the flat figures, 1e-5 relative for forward values and 1e-4 relative for gradients.
+"""
+import numpy as np
+import pytest
+
+from tests._metrics import abs_or_rel, covariance_condition
+
+pytestmark = [pytest.mark.gpu, pytest.mark.timeout(600)]
+
+
+def _say(test, **figures):
+    print("[full size] %s: %s" % (test, ", ".join("%s=%s" % (k, ("%.6g" % v) if isinstance(v, float) else v) for k, v in figures.items())))
+
+
+def test_chain_all_64Mi_problems(gpu, oracle):
+    import torch
+
+    from xyz_autodiff_cuda_amd import chain, rng
+
+    n, piece = 64 * 1024 * 1024, 8 * 1024 * 1024
+    ins = [torch.empty(n, dtype=torch.float32, device=gpu) for _ in range(6)]
+    rng.chain_inputs_(ins, seed=1234)
+    outs = chain.forward_backward(ins)
+    torch.cuda.synchronize()
+    value_ok = grads_ok = 0
+    # largest error (the testers' min(abs, rel)) of the value, of anything where cond(Sigma) <= e^2, and of
+    # anything divided by max(1, cond(Sigma)); against the exact answer (fp64) and against the fp32 oracle
+    worst = {ref: {"value": 0.0, "well_conditioned": 0.0, "scaled": 0.0} for ref in ("fp64", "fp32")}
+    closest = 0.0
+    for lo in range(0, n, piece):
+        sample = [t[lo:lo + piece].cpu().numpy() for t in ins]
+        got = np.stack([o[lo:lo + piece].cpu().numpy() for o in outs])
+        assert np.isfinite(got).all()
+        ref32 = oracle.chain_soa(sample, np.float32)
+        ref64 = oracle.chain_soa(sample, np.float64)
+        kappa = np.maximum(1.0, covariance_condition(sample[0], sample[1]))
+        e64 = abs_or_rel(got, ref64)
+        for name, e in (("fp64", e64), ("fp32", abs_or_rel(got, ref32))):
+            w = worst[name]
+            w["value"] = max(w["value"], (e[0] / kappa).max())
+            w["well_conditioned"] = max(w["well_conditioned"], e[:, kappa <= 7.4].max(initial=0.0))
+            w["scaled"] = max(w["scaled"], (e / kappa).max())
+        closest = max(closest, e64.max() / abs_or_rel(ref32, ref64).max())
+        value_ok += int((e64[0] <= 1e-5).sum())
+        grads_ok += int((e64[1:] <= 1e-4).all(axis=0).sum())
+    flat = {"value_within_1e-5": value_ok / n, "all_gradients_within_1e-4": grads_ok / n}
+    _say("chain 64 Mi", **{"%s_vs_%s" % (k, ref): v for ref in worst for k, v in worst[ref].items()},
+         distance_to_fp64_over_the_fp32_oracles=closest, **flat)
+    message = (worst, closest, flat)
+    # against the exact answer: 1e-5 where the covariance is well conditioned, 1e-5 x cond(Sigma) in general (the
+    # reference's own fp32 formulas lose that factor in det = ac - b^2, for q and hence the value as well)
+    assert worst["fp64"]["well_conditioned"] < 1e-5 and worst["fp64"]["scaled"] < 1e-5, message
+    # against another fp32 evaluation: each of the two may be that far from the exact answer
+    assert worst["fp32"]["well_conditioned"] < 2e-5 and worst["fp32"]["scaled"] < 2e-5, message
+    assert closest <= 2.0, message  # and never farther from it than twice the fp32 oracle's own distance
+    # the flat figures: every value within 1e-5 of the exact one; all six gradients within 1e-4 wherever
+    # cond(Sigma) x 6e-8 leaves room for it, which is all but a sliver of U(-2, 1) x U(-2, 1)
+    assert flat["value_within_1e-5"] == 1.0, message
+    assert flat["all_gradients_within_1e-4"] > 0.9999, message
+
+
+@pytest.mark.parametrize("strategy", ["auto", "wave_lds"])
+@pytest.mark.parametrize("num_slots", [64, 4096, 262144])
+def test_accumulation_16Mi_threads(gpu, oracle, num_slots, strategy):
+    import torch
+
+    from xyz_autodiff_cuda_amd import accumulate, rng
+
+    n = 16 * 1024 * 1024
+    ins = [torch.empty(n, dtype=torch.float32, device=gpu) for _ in range(6)]
+    rng.chain_inputs_(ins, seed=1234)
+    slot = torch.empty(n, dtype=torch.int32, device=gpu)
+    accumulate.zipf_(slot, seed=1234, stream_id=10, num_slots=num_slots)
+    grads = torch.zeros(num_slots, 6, dtype=torch.float32, device=gpu)
+    accumulate.accumulate_chain_gradients(ins, slot, grads, strategy)
+    torch.cuda.synchronize()
+    got = grads.cpu().numpy().astype(np.float64)
+    inputs = [t.cpu().numpy() for t in ins]
+    slots = slot.cpu().numpy()
+    assert slots.min() >= 0 and slots.max() < num_slots
+    sums, mass = oracle.accumulate_chain(inputs, slots, num_slots, chain_in_double=True)
+    g = oracle.chain_soa(inputs, np.float64)[1:]
+    kappa = np.maximum(1.0, covariance_condition(inputs[0], inputs[1]))
+    kmass = np.stack([np.bincount(slots, weights=kappa * np.maximum(1.0, np.abs(g[k])), minlength=num_slots) for k in range(6)], axis=1)
+    err = np.abs(got - sums)
+    excess = err / (1e-4 * mass + 1e-5 * kmass + 1e-30)
+    touched = mass > 0
+    flat = {"sums_within_1e-4_of_their_value": float((err[touched] <= 1e-4 * np.abs(sums[touched])).mean()),
+            "sums_within_1e-4_of_their_mass": float((err[touched] <= 1e-4 * mass[touched]).mean())}
+    _say("accumulate %d slots, %s" % (num_slots, strategy), worst_error_over_bound=float(excess.max()),
+         worst_error_over_mass=float((err[touched] / mass[touched]).max()), **flat)
+    assert excess.max() <= 1.0, (float(excess.max()), np.unravel_index(excess.argmax(), excess.shape), flat)
+    assert np.all(got[~touched] == 0.0)
+
+
+def _splat_case(gpu, oracle, G, W, H, scale_px):
+    import torch
+
+    from xyz_autodiff_cuda_amd import splat
+
+    target = splat.synthetic_target(G, W, H, seed=77, scale_px=scale_px, noise=0.02)
+    params, depth = splat.synthetic_scene(G, W, H, seed=1234, scale_px=scale_px)
+    ctx = splat.SplatContext(W, H, G)
+    image, grads, loss = ctx.step(params, depth, target)
+    torch.cuda.synchronize()
+    stats = ctx.stats(longest_list=True)
+    ctx.close()
+    hp, hd, ht = params.cpu().numpy(), depth.cpu().numpy(), target.cpu().numpy()
+    got_image, got = image.cpu().numpy(), grads.cpu().numpy().astype(np.float64)
+    del image, grads, target
+    assert np.isfinite(got_image).all() and np.isfinite(got).all()
+
+    o32 = oracle.splat_step(W, H, hp, hd, ht, np.float32)
+    # integer work: the same pairs and the same longest list as the fp32 oracle
+    assert stats["pairs"] == o32["pairs"] and stats["longest_list"] == o32["longest_list"], (stats, o32["pairs"], o32["longest_list"])
+    # fp64 on the tile rectangles of the fp32 projection: a 3-sigma box that ends within rounding of a tile
+    # edge would otherwise be binned differently and the two scenes would differ by whole (tile, Gaussian) pairs
+    o64 = oracle.splat_step(W, H, hp, hd, ht, np.float64, rects_in=o32["rects"], want_bounds=True)
+    assert o64["pairs"] == o32["pairs"]
+    # the image: 1e-5, plus what an fp32 evaluation may differ by where the 1e-4 stop can fall either way
+    image_excess = np.abs(got_image - o64["image"]) / (1e-5 + o64["image_bound"])
+    image_err = {"vs_fp32": float(np.abs(got_image - o32["image"]).max()), "vs_fp64": float(np.abs(got_image - o64["image"]).max()),
+                 "over_bound": float(image_excess.max())}
+    loss_err = {"vs_fp32": abs(loss - o32["loss"]) / o32["loss"], "vs_fp64": abs(loss - o64["loss"]) / o64["loss"]}
+
+    err = np.abs(got - o64["grads"])
+    tolerance = 1e-4 * o64["grad_mass"] + o64["grad_bound"] + 1e-30
+    excess = err / tolerance
+    within = (excess <= 1.0).all(axis=0)
+    nonzero = np.abs(o64["grads"]).max(axis=0) > 0
+    flat_gradients = (err <= 1e-4 * np.abs(o64["grads"])).all(axis=0)
+    oracle_excess = np.abs(o32["grads"].astype(np.float64) - o64["grads"]) / tolerance
+    figures = {
+        "pairs": int(stats["pairs"]), "longest_list": int(stats["longest_list"]),
+        "image_err_vs_fp32": image_err["vs_fp32"], "image_err_vs_fp64": image_err["vs_fp64"], "image_err_over_bound": image_err["over_bound"],
+        "loss_rel_err_vs_fp64": loss_err["vs_fp64"],
+        "gaussians_within_mass_bound": float(within.mean()), "worst_error_over_bound": float(excess.max()),
+        "fp32_oracle_worst_error_over_bound": float(oracle_excess.max()),
+        "median_bound_over_gradient": float(np.median((tolerance / (np.abs(o64["grads"]) + 1e-300))[:, nonzero])),
+        "gaussians_with_all_gradients_within_1e-4_relative": float(flat_gradients[nonzero].mean()),
+        "fp32_oracle_same_figure": float((np.abs(o32["grads"].astype(np.float64) - o64["grads"]) <= 1e-4 * np.abs(o64["grads"])).all(axis=0)[nonzero].mean()),
+        "pixels_within_1e-5": float((np.abs(got_image - o64["image"]) <= 1e-5).mean()),
+    }
+    _say("splat %d Gaussians %dx%d" % (G, W, H), **figures)
+    assert image_err["over_bound"] <= 1.0, (image_err, figures)
+    assert figures["pixels_within_1e-5"] > 0.9999, figures
+    assert loss_err["vs_fp32"] <= 1e-6 and loss_err["vs_fp64"] <= 1e-6, (loss_err, figures)
+    worst = np.unravel_index(excess.argmax(), excess.shape)
+    assert within.all(), ("Gaussians outside |gpu - fp64| <= 1e-4 mass + bound: %d of %d; worst row %d, Gaussian %d" %
+                          (int((~within).sum()), G, worst[0], worst[1]), figures)
+    return figures
+
+
+def test_splat_exactly_10k_gaussians_512(gpu, oracle):
+    figures = _splat_case(gpu, oracle, 10_000, 512, 512, (1.0, 20.0))
+    assert 100_000 < figures["pairs"] < 400_000
+
+
+def test_splat_exactly_200k_gaussians_2048(gpu, oracle):
+    figures = _splat_case(gpu, oracle, 200_000, 2048, 2048, (0.5, 40.0))
+    assert 4_000_000 < figures["pairs"] < 12_000_000 and figures["longest_list"] < 5000

@@ -239,3 +239,77 @@ def test_single_tile_scene_matches_an_independent_autograd_renderer(oracle):
     want = p.grad.numpy()
     scale = np.abs(want).max(axis=1, keepdims=True)
     assert np.all(np.abs(out["grads"] - want) <= 1e-9 * scale + 1e-14), np.abs(out["grads"] - want).max()
+
+
+# ---- the error bound the full-size GPU tests rest on (oracle_splat_step_ex: grad_mass, grad_bound, image_bound) ----
+
+BOUND_SCENES = [  # G, W, H, scale range in px, opacity shift, seed
+    (3000, 256, 192, (1.0, 20.0), 0.0, 1),   # the 10 000-Gaussian recipe, smaller
+    (6000, 256, 256, (0.5, 40.0), 0.0, 2),   # the 200 000-Gaussian recipe: anisotropic up to cond(Sigma) = 6400
+    (1500, 48, 48, (4.0, 16.0), 3.0, 3),     # opaque stacks: most pixels stop long before the end of their list
+    (4000, 320, 200, (0.5, 40.0), 1.5, 4),
+]
+
+
+def _bounded_pair(oracle, G, W, H, scale, shift, seed):
+    from tests._scenes import random_scene
+
+    params, depth = random_scene(G, W, H, seed=seed, scale_px=scale)
+    params[8] += shift
+    target = np.random.default_rng(seed + 1).uniform(0, 1, (H, W, 3)).astype(np.float32)
+    o32 = oracle.splat_step(W, H, params, depth, target, np.float32)
+    o64 = oracle.splat_step(W, H, params, depth, target, np.float64, rects_in=o32["rects"], want_bounds=True)
+    return params, depth, target, o32, o64
+
+
+@pytest.mark.parametrize("scene", BOUND_SCENES)
+def test_fp32_evaluation_stays_within_the_first_order_bound(oracle, scene):
+    """An independent fp32 evaluation of the step (the fp32 oracle: other summation order, library
+    exp and sincos) must lie within 1e-4 mass + bound of the fp64 one for every gradient of every
+    Gaussian, and within 1e-5 + image_bound at every pixel."""
+    G, W, H = scene[:3]
+    _, _, _, o32, o64 = _bounded_pair(oracle, *scene)
+    assert o64["pairs"] == o32["pairs"]
+    tolerance = 1e-4 * o64["grad_mass"] + o64["grad_bound"] + 1e-30
+    excess = np.abs(o32["grads"].astype(np.float64) - o64["grads"]) / tolerance
+    assert excess.max() <= 1.0, (excess.max(), np.unravel_index(excess.argmax(), excess.shape))
+    image_excess = np.abs(o32["image"].astype(np.float64) - o64["image"]) / (1e-5 + o64["image_bound"])
+    assert image_excess.max() <= 1.0
+    assert np.all(o64["grad_mass"] >= np.abs(o64["grads"]) * (1 - 1e-9))  # a sum of magnitudes bounds the sum
+
+
+@pytest.mark.parametrize("scene,median_limit,mistake", [(BOUND_SCENES[0], 1e-2, 0.05), (BOUND_SCENES[1], 1e-1, 0.25)])
+def test_the_bound_is_not_vacuous(oracle, scene, median_limit, mistake):
+    """It must catch a real mistake: a relative error of 5 % in the gradients (25 % where covariances reach
+    cond(Sigma) = 6400 and fp32 itself is that poor) is outside it for most entries, and it is small against
+    the gradients themselves; for colours, which take no part in the ill-conditioned inverse, everywhere."""
+    params, depth, target, o32, o64 = _bounded_pair(oracle, *scene)
+    tolerance = 1e-4 * o64["grad_mass"] + o64["grad_bound"] + 1e-30
+    live = np.abs(o64["grads"]) > 1e-12
+    relative = tolerance / np.abs(o64["grads"] + 1e-300)
+    assert np.median(relative[live]) < median_limit, np.median(relative[live])
+    caught = (np.abs(mistake * o64["grads"]) > tolerance)[live]
+    assert caught.mean() > 0.5, caught.mean()
+    assert np.percentile(relative[5:8][live[5:8]], 90) < 2e-2, np.percentile(relative[5:8][live[5:8]], 90)
+
+
+def test_bounds_do_not_change_the_step_and_rectangles_round_trip(oracle):
+    from tests._scenes import random_scene
+
+    G, W, H = 800, 128, 96
+    params, depth = random_scene(G, W, H, seed=5, scale_px=(1.0, 15.0))
+    target = np.random.default_rng(6).uniform(0, 1, (H, W, 3)).astype(np.float32)
+    plain = oracle.splat_step(W, H, params, depth, target, np.float64)
+    again = oracle.splat_step(W, H, params, depth, target, np.float64, rects_in=plain["rects"], want_bounds=True)
+    assert np.array_equal(plain["rects"], again["rects"]) and plain["pairs"] == again["pairs"]
+    assert np.array_equal(plain["image"], again["image"])
+    scale = np.abs(plain["grads"]).max()
+    assert np.abs(plain["grads"] - again["grads"]).max() <= 1e-12 * scale  # thread partition differs run to run
+    assert abs(plain["loss"] - again["loss"]) <= 1e-12 * plain["loss"]
+    # rectangles given from outside are used as given: an emptied rectangle removes the Gaussian
+    rects = plain["rects"].copy()
+    rects[:10] = (1, 1, 0, 0)
+    fewer = oracle.splat_step(W, H, params, depth, target, np.float64, rects_in=rects)
+    x0, y0, x1, y1 = plain["rects"][:10].T
+    assert fewer["pairs"] == plain["pairs"] - int((np.maximum(0, x1 - x0 + 1) * np.maximum(0, y1 - y0 + 1)).sum())
+    assert np.all(fewer["grads"][:, :10] == 0.0)

@@ -197,7 +197,9 @@ def test_repeated_steps_are_independent(gpu):
     torch.cuda.synchronize()
     assert torch.equal(first[0], again[0])
     scale = first[1].abs().amax(dim=0) + 1e-20
-    assert float(((first[1] - again[1]).abs() / scale).max()) < 1e-5  # atomics: order varies, values do not pile up
+    # atomics: the order of the per-tile sums varies from run to run (1e-4 relative is the figure allowed for
+    # that); the values do not pile up from call to call
+    assert float(((first[1] - again[1]).abs() / scale).max()) < 1e-4
     assert abs(first[2] - again[2]) <= 1e-9 * first[2]
     ctx.close()
 

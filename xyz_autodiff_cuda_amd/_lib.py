@@ -34,8 +34,6 @@ SIGNATURES = {
     "xad_abi_version": [],
     "xad_source_digest": [],
     "xad_chain_forward_backward_f32": [_sz] + [_vp] * 13 + [_vp],
-    "xad_chain_forward_backward_f32_layout": [_sz] + [_vp] * 13 + [_int, _vp],
-    "xad_stream_copy_f32": [_sz, _vp, _vp, _vp],
     "xad_host_chain_forward_backward_f32": [_sz] + [_vp] * 13 + [_int],
     "xad_host_chain_forward_backward_f64": [_sz] + [_vp] * 13 + [_int],
     "xad_accumulate_chain_gradients_f32": [_int, _sz] + [_vp] * 8 + [_int, _vp],
@@ -67,9 +65,6 @@ SIGNATURES = {
     "xad_linreg_sgd_f64": [_sz, _vp, _vp, _vp, _vp, _int, _int, ctypes.c_double, ctypes.c_double, _u64, _vp, _vp],
     "xad_linreg_sgd_f64_static": [_sz, _vp, _vp, _vp, _vp, _int, _int, ctypes.c_double, ctypes.c_double, _u64, _vp, _vp],
     "xad_host_linreg_gradient_f64": [_sz, _sz, _vp, _vp, _vp, _vp, _vp, _vp],
-    "xad_probe_chain_store_policy": [_int, _sz] + [_vp] * 13 + [_vp],
-    "xad_chain_kernel_resources": [_vp],
-    "xad_probe_lds_atomic_cycles": [_int, _int, ctypes.POINTER(ctypes.c_double)],
     "xad_rng_zipf_i32": [_vp, _sz, _u64, _u64, _int, ctypes.c_double, _vp],
     "xad_rng_uniform_f32": [_vp, _sz, _u64, _u64, _flt, _flt, _vp],
     "xad_rng_normal_f32": [_vp, _sz, _u64, _u64, _flt, _flt, _vp],

@@ -67,22 +67,3 @@ def zipf_(slot, seed, stream_id, num_slots, exponent=1.1):
                                           torch.cuda.current_stream(slot.device).cuda_stream)
     _lib.check(st, "xad_rng_zipf_i32")
     return slot
-
-
-LDS_PROBE_ELEMENTS = ("f32", "f64", "u32", "u64")
-LDS_PROBE_PATTERNS = ("64_distinct", "one_address", "16_lanes_share", "8_lanes_per_address", "stride_6")
-
-
-def lds_atomic_cycles():
-    """Measures LDS atomic-add cost: {element: {pattern: cycles per wavefront instruction}}."""
-    import ctypes
-
-    lib = _lib.load()
-    out = {}
-    for e, ename in enumerate(LDS_PROBE_ELEMENTS):
-        out[ename] = {}
-        for p, pname in enumerate(LDS_PROBE_PATTERNS):
-            c = ctypes.c_double(0.0)
-            _lib.check(lib.xad_probe_lds_atomic_cycles(e, p, ctypes.byref(c)), "xad_probe_lds_atomic_cycles")
-            out[ename][pname] = c.value
-    return out

@@ -23,14 +23,12 @@ def _require_cuda_f32(t, name, n):
         raise ValueError("%s must be a contiguous float32 tensor of %d elements" % (name, n))
 
 
-def forward_backward(inputs, outputs=None, stream=None, problems_per_lane=None):
+def forward_backward(inputs, outputs=None, stream=None):
     """Runs the graph for every problem on the GPU.
 
     inputs:  six float32 CUDA tensors (sx, sy, theta, o, px, py) of equal length n.
     outputs: optional seven preallocated float32 CUDA tensors; allocated if None.
     stream:  torch.cuda.Stream to launch on (default: the current stream).
-    problems_per_lane: None for the library default, or 1 / 4 to pick the
-             lane-to-address mapping explicitly (4 = 16-byte accesses).
     Returns the seven output tensors (w, d_sx, d_sy, d_theta, d_o, d_px, d_py).
     """
     import torch
@@ -50,43 +48,9 @@ def forward_backward(inputs, outputs=None, stream=None, problems_per_lane=None):
     s = stream if stream is not None else torch.cuda.current_stream(inputs[0].device)
     ptrs = [t.data_ptr() for t in inputs] + [t.data_ptr() for t in outputs]
     with torch.cuda.device(inputs[0].device):
-        if problems_per_lane is None:
-            status = lib.xad_chain_forward_backward_f32(n, *ptrs, s.cuda_stream)
-        else:
-            status = lib.xad_chain_forward_backward_f32_layout(n, *ptrs, int(problems_per_lane), s.cuda_stream)
+        status = lib.xad_chain_forward_backward_f32(n, *ptrs, s.cuda_stream)
     _lib.check(status, "xad_chain_forward_backward_f32")
     return outputs
-
-
-STORE_POLICIES = {"write_through": 0, "plain": 1, "non_temporal": 2}
-
-
-def store_policy_probe(inputs, outputs, policy, stream=None):
-    """The default kernel with another store policy (see xad_probe_chain_store_policy); same results."""
-    import torch
-
-    lib = _lib.load()
-    n = inputs[0].numel()
-    for t, name in zip(list(inputs) + list(outputs), INPUT_NAMES + OUTPUT_NAMES):
-        _require_cuda_f32(t, name, n)
-    s = stream if stream is not None else torch.cuda.current_stream(inputs[0].device)
-    ptrs = [t.data_ptr() for t in inputs] + [t.data_ptr() for t in outputs]
-    with torch.cuda.device(inputs[0].device):
-        status = lib.xad_probe_chain_store_policy(STORE_POLICIES[policy] if isinstance(policy, str) else int(policy), n, *ptrs,
-                                                  s.cuda_stream)
-    _lib.check(status, "xad_probe_chain_store_policy")
-    return outputs
-
-
-def kernel_resources():
-    """Registers, scratch, LDS and residency of the default kernel, as the loaded code object and the device report them."""
-    import ctypes
-
-    out = (ctypes.c_int * 5)()
-    _lib.check(_lib.load().xad_chain_kernel_resources(ctypes.cast(out, ctypes.c_void_p)), "xad_chain_kernel_resources")
-    vgprs, scratch, lds, lanes, blocks = list(out)
-    return {"vgprs_per_lane": vgprs, "scratch_bytes_per_lane": scratch, "lds_bytes_per_block": lds, "lanes_per_block": lanes,
-            "blocks_per_cu": blocks, "wavefronts_per_simd": blocks * lanes // 64 // 4}
 
 
 def host_forward_backward(inputs, dtype=np.float32, num_threads=0):
@@ -107,17 +71,3 @@ def host_forward_backward(inputs, dtype=np.float32, num_threads=0):
     status = fn(n, *[a.ctypes.data for a in arrays], *[a.ctypes.data for a in outs], int(num_threads))
     _lib.check(status, fn.__name__)
     return outs
-
-
-def stream_copy(src, dst, stream=None):
-    """dst[:] = src on the GPU with the chain kernel's access pattern (calibration yardstick)."""
-    import torch
-
-    n = src.numel()
-    _require_cuda_f32(src, "src", n)
-    _require_cuda_f32(dst, "dst", n)
-    s = stream if stream is not None else torch.cuda.current_stream(src.device)
-    with torch.cuda.device(src.device):
-        st = _lib.load().xad_stream_copy_f32(n, src.data_ptr(), dst.data_ptr(), s.cuda_stream)
-    _lib.check(st, "xad_stream_copy_f32")
-    return dst

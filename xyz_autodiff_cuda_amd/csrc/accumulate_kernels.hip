@@ -41,6 +41,10 @@ struct AccumulateArgs {
     unsigned spill_offset;
     // copies of a small table, so that lanes sharing a slot do not share an LDS address
     int replicas;
+    // a table smaller than the slot count: rows claimed on first use (1) or owned by the first slots (0)
+    int claim_rows;
+    // slots below this are the ones kept in `replicas` copies (negative: all)
+    int hot_rows;
 };
 
 // Which part a block serves, the rows of its table and where they live in the global array.
@@ -62,7 +66,8 @@ __global__ void __launch_bounds__(kBlock) accumulate_kernel(AccumulateArgs a) {
     extern __shared__ __attribute__((aligned(16))) float lds[];
     const Part part(a);
     BlockAccumulator<float, kWidth, S, Peel, 4, TableT, Spill> acc(lds, a.capacity, a.grads + part.index * kWidth,
-                                                                   part.rows, part.parts * kWidth, a.replicas);
+                                                                   part.rows, part.parts * kWidth, a.replicas,
+                                                                   a.claim_rows != 0, a.hot_rows);
     if constexpr (Spill) acc.use_spill_staging(reinterpret_cast<char*>(lds) + a.spill_offset);
 
     const std::size_t begin = static_cast<std::size_t>(blockIdx.x >> a.part_shift) * a.per_block;
@@ -114,7 +119,7 @@ __global__ void __launch_bounds__(kBlock) accumulate_leaf_kernel(AccumulateArgs 
     using Acc = BlockAccumulator<float, kWidth, S, 0, 4, TableT>;
     extern __shared__ __attribute__((aligned(16))) float lds[];
     const Part part(a);
-    Acc acc(lds, a.capacity, a.grads + part.index * kWidth, part.rows, part.parts * kWidth, a.replicas);
+    Acc acc(lds, a.capacity, a.grads + part.index * kWidth, part.rows, part.parts * kWidth, a.replicas, true, a.hot_rows);
 
     const std::size_t begin = static_cast<std::size_t>(blockIdx.x >> a.part_shift) * a.per_block;
     const std::size_t end = begin + a.per_block < a.n ? begin + a.per_block : a.n;
@@ -200,15 +205,46 @@ extern "C" int xad_accumulate_chain_gradients_f32(int strategy, std::size_t n, c
                                                   void* stream) {
     const char* who = "xad_accumulate_chain_gradients_f32";
     if (n == 0) return XAD_OK;
-    AccumulateArgs a{{sx, sy, theta, o, px, py}, slot, grads, n, 0, num_slots, 0, 0, 0, 1};
+    AccumulateArgs a{{sx, sy, theta, o, px, py}, slot, grads, n, 0, num_slots, 0, 0, 0, 1, 1, -1};
     for (int k = 0; k < 6; ++k) XAD_REQUIRE(a.in[k], "%s: input array %d is null", who, k);
     XAD_REQUIRE(slot && grads, "%s: slot or grads is null", who);
     XAD_REQUIRE(num_slots > 0, "%s: num_slots must be positive, got %d", who, num_slots);
 
     // Strategy AUTO: the LDS table.  With small tables replicated (below) it is the fastest at every
-    // slot count measured, 1 to 262 144; the wavefront pre-reduction stays selectable.
-    if (strategy == XAD_ACCUMULATE_AUTO) strategy = XAD_ACCUMULATE_LDS;
-
+    // slot count measured, 1 to 262 144; the wavefront pre-reduction stays selectable.  Beyond what one
+    // fp64 table holds, AUTO gives the rows to the first slots and sends the rest through the coalesced
+    // spill: one walk over the inputs, no tags, no probing.
+    constexpr std::size_t kSpillBytes = BlockAccumulator<float, kWidth>::spill_bytes(kBlock);
+    constexpr std::size_t kRowBytes = kWidth * sizeof(double);
+    // The first kHotRows slots are kept in several copies (lane l adds into copy l % copies): under a skewed
+    // law over the slot index they take most of the adds, and lanes that share an LDS address serialise.
+    constexpr int kHotRows = 64;
+    if (strategy == XAD_ACCUMULATE_AUTO) {
+        if (static_cast<std::size_t>(num_slots) * kRowBytes > 144 * 1024) {
+            const int rows = static_cast<int>((kMaxLdsBytes - kSpillBytes) / kRowBytes);
+            a.capacity = rows;
+            a.claim_rows = 0;
+            // Measured at 16 Mi threads, Zipf(1.1): 8 copies of the 32 hottest rows up to 16 384 slots (4096 slots
+            // 0.162 ms against 0.181 without copies), 4 copies beyond, where the rows the copies take away
+            // from the other slots cost more (262 144 slots: 0.241 ms with 4 copies, 0.257 with 8, 0.265 with none).
+            a.replicas = num_slots <= 32768 ? 8 : 4;
+            a.hot_rows = 32;
+            a.spill_offset = static_cast<unsigned>(static_cast<std::size_t>(rows) * kRowBytes);
+            return launch(accumulate_kernel<Strategy::LdsAtomics, 0, double, true>, a, a.spill_offset + kSpillBytes, 1, stream);
+        }
+        if (num_slots > kHotRows) {
+            // one fp64 table for every slot, the hot rows in as many copies as the LDS of a CU still holds
+            a.hot_rows = kHotRows;
+            a.replicas = 16;
+            while (a.replicas > 1 &&
+                   static_cast<std::size_t>(BlockAccumulator<float, kWidth>::rows_for(num_slots, a.replicas, kHotRows)) * kRowBytes > kMaxLdsBytes)
+                a.replicas /= 2;
+            a.capacity = BlockAccumulator<float, kWidth>::rows_for(num_slots, a.replicas, kHotRows);
+            const std::size_t lds = static_cast<std::size_t>(a.capacity) * kRowBytes;
+            return launch(accumulate_kernel<Strategy::LdsAtomics, 0, double>, a, lds, lds <= 72 * 1024 ? 2 : 1, stream);
+        }
+        strategy = XAD_ACCUMULATE_LDS;
+    }
     // LDS table (at most 144 KiB): fp64 rows for every slot if they fit; if they fit in two
     // tables, the slots are dealt to two sets of blocks that each walk all threads (the inputs
     // are read twice, but ds_add_f64 is that much faster than ds_add_f32); otherwise fp32 rows
@@ -234,9 +270,9 @@ extern "C" int xad_accumulate_chain_gradients_f32(int strategy, std::size_t n, c
     a.capacity = direct ? static_cast<int>(cells / kWidth) : (tagged_f64 ? 2048 : 4096);
     if (direct && staged && a.part_shift == 0) {
         // a small table is replicated: up to 16 copies within 48 KiB (two blocks per CU stay resident)
-        const std::size_t copy_rows = static_cast<std::size_t>(BlockAccumulator<float, kWidth>::replica_rows(num_slots));
+        const std::size_t copy_rows = static_cast<std::size_t>(num_slots | 1);
         while (a.replicas < 16 && copy_rows * (a.replicas * 2) * kWidth * cell <= 48 * 1024) a.replicas *= 2;
-        if (a.replicas > 1) a.capacity = static_cast<int>(copy_rows) * a.replicas;
+        if (a.replicas > 1) a.capacity = BlockAccumulator<float, kWidth>::rows_for(num_slots, a.replicas, num_slots);
     }
     std::size_t lds = static_cast<std::size_t>(a.capacity) * kWidth * cell + (direct ? 0 : a.capacity * 4u);
     if (lds < 16) lds = 16;

@@ -252,6 +252,35 @@ __device__ __forceinline__ Staged stage_record(const Record* __restrict__ record
     return s;
 }
 
+// List entries that cannot be seen from a tile.  The binning rectangle is the 3-sigma box of the
+// Gaussian's own axes-aligned extent, so a rotated, elongated Gaussian is listed in corner tiles that
+// its ellipse never comes near (about a fifth of all pairs when scales span 0.5 to 40 pixels).  Such
+// an entry is recognised when its record is staged: the minimum of q over the tile's pixel centres
+// is bounded from below by the minimum over their bounding box, which for a convex quadratic whose
+// centre lies outside the box is attained on one of the four edges.  If even there alpha stays below
+// kNegligibleAlpha, the entry is left out of the compositing loops of this tile, forward and backward
+// alike: it would change a pixel by less than 1e-8 (an fp32 ulp of 0.5 is 6e-8).  Lists and pair
+// counts are not affected.  Comparisons with NaN are false, so an odd record is kept.
+constexpr float kNegligibleAlpha = 1e-8f;
+
+__device__ __forceinline__ bool negligible_in_tile(const Staged& s, float tile_x, float tile_y) {
+    const float x0 = tile_x - s.cx, x1 = x0 + static_cast<float>(kTile - 1);
+    const float y0 = tile_y - s.cy, y1 = y0 + static_cast<float>(kTile - 1);
+    float q_min = 0.f;
+    if (!(x0 <= 0.f && x1 >= 0.f && y0 <= 0.f && y1 >= 0.f)) {
+        auto along_x = [&](float y) {  // min over x in [x0, x1] of a x^2 + 2 b x y + c y^2
+            const float x = __builtin_fminf(__builtin_fmaxf(-s.b * y / s.a, x0), x1);
+            return ::fmaf(::fmaf(s.a, x, 2.f * s.b * y), x, s.c * y * y);
+        };
+        auto along_y = [&](float x) {
+            const float y = __builtin_fminf(__builtin_fmaxf(-s.b * x / s.c, y0), y1);
+            return ::fmaf(::fmaf(s.c, y, 2.f * s.b * x), y, s.a * x * x);
+        };
+        q_min = __builtin_fminf(__builtin_fminf(along_x(y0), along_x(y1)), __builtin_fminf(along_y(x0), along_y(x1)));
+    }
+    return s.alpha0 * math::fp32::exp2_raw(-kHalfLog2e * q_min) < kNegligibleAlpha;
+}
+
 __device__ __forceinline__ std::uint32_t wave_max(std::uint32_t v) {
     // 64-lane maximum through the LDS crossbar-free DPP path: rows, then row heads
     auto step = [](std::uint32_t x, auto ctrl) {
@@ -298,12 +327,19 @@ __global__ void __launch_bounds__(kChunk) render_forward_kernel(
         used[p] = 0;
     }
 
+    const float tile_x = static_cast<float>((tile % tiles_x) * kTile), tile_y = static_cast<float>((tile / tiles_x) * kTile);
     for (std::uint32_t base = first; base < last; base += kChunk) {
         __syncthreads();
-        if (base + lane < last) staged[lane] = stage_record(records, sorted_ids[base + lane]);
+        bool visible = false;
+        if (base + lane < last) {
+            const Staged mine = stage_record(records, sorted_ids[base + lane]);
+            staged[lane] = mine;
+            visible = !negligible_in_tile(mine, tile_x, tile_y);
+        }
         __syncthreads();
-        const int count = __builtin_amdgcn_readfirstlane(static_cast<int>(last - base < kChunk ? last - base : kChunk));
-        for (int j = 0; j < count; ++j) {
+        // the staged entries that can be seen from this tile, front to back
+        for (std::uint64_t todo = accumulate::wave::ballot(visible); todo != 0; todo &= todo - 1) {
+            const int j = __builtin_ctzll(todo);
             const Staged r = staged[j];
             // exponent of the falloff as a polynomial in dx: (a_s dx + e) dx + f
             const float dy = py - r.cy;
@@ -423,6 +459,7 @@ __global__ void __launch_bounds__(kChunk) render_backward_kernel(
     // Row sums wait here until a group of kPark list entries is complete.  Small on purpose: LDS per
     // block, not registers, is what limits the number of resident wavefronts.
     __shared__ float parked[kPark][4][9];  // [list entry within its group][row of 16 lanes][value]
+    __shared__ int parked_entry[kPark];    // which staged entry that is
 
     const int tile = tile_of_block(blockIdx.x, tiles);
     if (tile >= tiles) return;
@@ -470,21 +507,28 @@ __global__ void __launch_bounds__(kChunk) render_backward_kernel(
     const int park_index = reduced_index(lane);
     const bool parks = !(lane & 2) || (lane & 15) == 2;
 
+    const float tile_x = static_cast<float>((tile % tiles_x) * kTile), tile_y = static_cast<float>((tile / tiles_x) * kTile);
     for (std::uint32_t chunk = (deepest + kChunk - 1) / kChunk; chunk-- > 0;) {
         const std::uint32_t chunk_first = chunk * kChunk;
         const int count = static_cast<int>(deepest - chunk_first < kChunk ? deepest - chunk_first : kChunk);
         __syncthreads();
+        bool visible = false;
         if (lane < count) {
             const std::uint32_t id = sorted_ids[first + chunk_first + lane];
             staged_id[lane] = id;
-            staged[lane] = stage_record(records, id);
+            const Staged mine = stage_record(records, id);
+            staged[lane] = mine;
+            visible = !negligible_in_tile(mine, tile_x, tile_y);  // the forward pass left the same entries out
         }
         __syncthreads();
 
-        // groups of up to kPark entries, back to front; all but the last-staged one are full
-        for (int group_end = count; group_end > 0;) {
-            const int group_first = (group_end - 1) / kPark * kPark;
-            for (int j = group_end - 1; j >= group_first; --j) {
+        // the staged entries that can be seen from this tile, back to front, in groups of up to kPark
+        std::uint64_t todo = accumulate::wave::ballot(visible);
+        while (todo != 0) {
+            int members = 0;
+            for (; todo != 0 && members < kPark; ++members) {
+                const int j = 63 - __builtin_clzll(todo);
+                todo &= ~(std::uint64_t(1) << j);
                 const std::uint32_t position = chunk_first + j;
                 const Staged r = staged[j];
                 // exponent of the falloff as a polynomial in dx: (a_s dx + e) dx + f
@@ -528,15 +572,15 @@ __global__ void __launch_bounds__(kChunk) render_backward_kernel(
                 const float sy = dy * m0;
                 const float v[9] = {sx, sy, ::fmaf(dx0, sx + m1, m2), dy * sx, dy * sy, colour[0], colour[1], colour[2], m0};
                 const float mine = reduce_scatter9(v, lane);
-                if (parks) parked[j - group_first][lane >> 4][park_index] = mine;
+                if (parks) parked[members][lane >> 4][park_index] = mine;
+                if (lane == 0) parked_entry[members] = j;
             }
-            const int members = group_end - group_first;
             __syncthreads();
             if (lane < members) {
                 float s[9];
 #pragma unroll
                 for (int k = 0; k < 9; ++k) s[k] = (parked[lane][0][k] + parked[lane][1][k]) + (parked[lane][2][k] + parked[lane][3][k]);
-                const Staged r = staged[group_first + lane];
+                const Staged r = staged[parked_entry[lane]];
                 const float g_q_scale = -0.5f * r.alpha0;
 #pragma unroll
                 for (int k = 0; k < 5; ++k) s[k] *= g_q_scale;
@@ -558,10 +602,9 @@ __global__ void __launch_bounds__(kChunk) render_backward_kernel(
                 const float value = parked[entry][0][field];
                 if (value != 0.f)
                     detail::atomic_add(
-                        record_grads + static_cast<std::size_t>(staged_id[group_first + entry]) * kRecordGradStride + field, value);
+                        record_grads + static_cast<std::size_t>(staged_id[parked_entry[entry]]) * kRecordGradStride + field, value);
             }
             __syncthreads();  // the next group parks into the same rows
-            group_end = group_first;
         }
     }
 }
