@@ -227,7 +227,8 @@ def splat_report(with_oracle, iters=30):
         target = splat.synthetic_target(G, W, H, seed=77, scale_px=scale, noise=0.02)
         params, depth = splat.synthetic_scene(G, W, H, seed=1234, scale_px=scale)
         start_params = params.clone()
-        ctx = splat.SplatContext(W, H, G, pair_capacity_hint=9_000_000 if G > 50_000 else 0)
+        # depths never change in this loop: say so, and an iteration never waits for the device
+        ctx = splat.SplatContext(W, H, G, pair_capacity_hint=9_000_000 if G > 50_000 else 0, depth_mode="static")
         m, v = torch.zeros_like(params), torch.zeros_like(params)
         image = torch.empty(H, W, 3, device=dev)
         grads = torch.empty(9, G, device=dev)

@@ -37,6 +37,7 @@ extern "C" {
 #define XAD_ERR_INVALID_ARGUMENT 1 /* null pointer, bad size, bad enum value    */
 #define XAD_ERR_HIP 2              /* a HIP runtime call or kernel launch failed */
 #define XAD_ERR_UNSUPPORTED 3      /* valid request this build cannot serve      */
+#define XAD_ERR_INCOMPLETE 5       /* an earlier asynchronous call came out incomplete (see xad_splat_step) */
 
 /* Text of the most recent error on this thread ("" if none). */
 const char* xad_last_error(void);
@@ -151,14 +152,31 @@ int xad_accumulate_chain_gradients_f32(int strategy, size_t n,
  *   target, image   device, height x width x 3 floats, interleaved RGB
  *   grads   device, 9 rows of G floats, overwritten
  *
- * The context owns all intermediate device buffers (records, pair lists, sort
- * workspace, per-pixel state); they grow when a step produces more (tile,
- * Gaussian) pairs than fit.  A step reads two words back (the pair count, which
- * sizes the sort, and whether any depth differs from the previous call's), so
- * calls synchronise with `stream` once; the order of the Gaussians by (depth,
- * index) is kept between calls and recomputed, with one more synchronisation,
- * only in a call whose depths differ.  One context serves one stream at a time
- * and belongs to the device that was current when it was created.
+ * The context owns all intermediate device buffers (records, tile lists, per-pixel
+ * state, binning workspace) in two allocations, one sized by (G, image), one by
+ * the capacity of the tile lists in (tile, Gaussian) pairs.  One context serves
+ * one stream at a time and belongs to the device that was current when it was
+ * created.
+ *
+ * When the host waits.  The tile lists are built on the device without any
+ * read-back (no sort; see csrc/splat_binning.hip).  The host looks at what the
+ * device found only
+ *   - in the first call after the lists were sized (creation, or enlargement):
+ *     did the pairs fit?  If not the lists are enlarged and the binning redone;
+ *   - in every call of the default depth mode, XAD_SPLAT_DEPTH_CHECKED: did any
+ *     depth change since the call that last ordered the Gaussians?  (The order by
+ *     (depth, index) is kept between calls; one changed bit reorders.)
+ *   - when the caller asks for the loss.
+ * A caller whose depths do not change sets XAD_SPLAT_DEPTH_STATIC (a promise:
+ * depth is read by the first call and assumed unchanged afterwards); one whose
+ * depths change all the time sets XAD_SPLAT_DEPTH_EVERY_STEP (the order is
+ * recomputed by every call, on the device).  In both modes a step with
+ * loss_out == NULL only queues work.  What such a call cannot report itself is
+ * reported by the next call that waits (a step with loss_out, xad_splat_get_stats):
+ * XAD_ERR_INCOMPLETE if a step produced more pairs than the lists held (its image
+ * and gradients lack the pairs that did not fit; the lists are enlarged at that
+ * point), XAD_ERR_INVALID_ARGUMENT if a depth changed under the static promise.
+ * The outputs of the call that returns such a status are themselves complete.
  */
 typedef struct xad_splat_context xad_splat_context;
 int xad_splat_create(int width, int height, int num_gaussians, size_t pair_capacity_hint,
@@ -168,19 +186,29 @@ void xad_splat_destroy(xad_splat_context* ctx);
 int xad_splat_forward(xad_splat_context* ctx, const float* params, const float* depth,
                       float* image, void* stream);
 /* Render, loss and gradients.  loss_out (host, may be NULL) receives the sum of
- * squared errors; passing it makes the call wait for the stream. */
+ * squared errors; passing it makes the call wait for the stream (and, should this
+ * very step not fit the lists, enlarge them and run it again). */
 int xad_splat_step(xad_splat_context* ctx, const float* params, const float* depth,
                    const float* target, float* image, float* grads, double* loss_out,
                    void* stream);
-/* Per-stage GPU times (events around project, scan+emit, sort, tile ranges,
- * render forward, render backward, parameter backward) are recorded by the next
- * calls when enabled; recording makes each call wait for the stream. */
+#define XAD_SPLAT_DEPTH_CHECKED 0
+#define XAD_SPLAT_DEPTH_STATIC 1
+#define XAD_SPLAT_DEPTH_EVERY_STEP 2
+int xad_splat_set_depth_mode(xad_splat_context* ctx, int mode);
+/* Per-stage GPU times (events around project, binning, render forward, render
+ * backward, parameter backward) are recorded by the next calls when enabled;
+ * recording makes each call wait for the stream. */
 int xad_splat_set_profiling(xad_splat_context* ctx, int enabled);
-/* Of the last call: number of (tile, Gaussian) pairs, longest tile list, and the
- * seven stage times in milliseconds (zeros unless profiling is enabled).  Any
- * output pointer may be NULL. */
-int xad_splat_get_stats(const xad_splat_context* ctx, uint64_t* pairs, uint32_t* longest_list,
-                        float* stage_ms);
+/* Of the last call: number of (tile, Gaussian) pairs, longest tile list (either
+ * makes the call wait for the device), and the five stage times in milliseconds
+ * (zeros unless profiling is enabled).  Any output pointer may be NULL. */
+int xad_splat_get_stats(xad_splat_context* ctx, uint64_t* pairs, uint32_t* longest_list, float* stage_ms);
+/* The tile lists of the last call, to host memory: tile t (row-major) holds
+ * gaussians[range_begin[t] .. range_end[t]), in compositing order.  range_begin and
+ * range_end: one entry per tile; gaussians (may be NULL): room for `capacity`
+ * entries, at least the pair count.  Waits for the device. */
+int xad_splat_get_lists(xad_splat_context* ctx, uint32_t* range_begin, uint32_t* range_end,
+                        uint32_t* gaussians, size_t capacity);
 
 /* Adam over structure-of-arrays parameters: `rows` rows of n floats each in
  * params, grads, m and v (device); row r uses row_learning_rates[r] (host).

@@ -56,7 +56,7 @@ XADI_EXPORT int xadi_chain_forward_backward_f32_layout(std::size_t n, const floa
     hipStream_t s = xad::as_stream(stream);
     const std::size_t groups = vector_ok ? n / 4 : 0;
     if (groups) {
-        hipLaunchKernelGGL(xad_chain::chain_quad_kernel, dim3(xad::blocks_for(groups, kQuadBlock)), dim3(kQuadBlock), 0, s,
+        hipLaunchKernelGGL(xad_chain::chain_quad_kernel<>, dim3(xad::blocks_for(groups, kQuadBlock)), dim3(kQuadBlock), 0, s,
                            buf, groups);
         XAD_HIP_TRY(hipGetLastError());
     }
@@ -93,7 +93,7 @@ XADI_EXPORT int xadi_stream_copy_f32(std::size_t n, const float* src, float* dst
     if (n == 0) return 0;
     XAD_REQUIRE(src && dst, "xadi_stream_copy_f32: null array");
     XAD_REQUIRE(n <= 0x7fffffffull * 64, "xadi_stream_copy_f32: n = %zu exceeds the grid limit", n);
-    hipLaunchKernelGGL(xad_chain::stream_copy_kernel, dim3(xad::blocks_for(n, kSingleBlock)), dim3(kSingleBlock), 0,
+    hipLaunchKernelGGL(xad_chain::stream_copy_kernel<>, dim3(xad::blocks_for(n, kSingleBlock)), dim3(kSingleBlock), 0,
                        xad::as_stream(stream), src, dst, n);
     XAD_HIP_TRY(hipGetLastError());
     return 0;

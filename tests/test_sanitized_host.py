@@ -53,7 +53,7 @@ def _corpus(directory):
 def test_host_tier_under_address_and_undefined_behaviour_sanitizers(tmp_path):
     exe = str(tmp_path / "sanitized_host")
     hip_include = os.path.join(os.path.dirname(os.path.dirname(os.environ.get("HIPCC", "/opt/rocm/bin/hipcc"))), "include")
-    cmd = [os.environ.get("CXX", "g++"), "-std=c++20", "-O1", "-g", "-fsanitize=address,undefined", "-fno-sanitize-recover=all",
+    cmd = [os.environ.get("CXX", "g++"), "-std=c++20", "-O0", "-g1", "-fsanitize=address,undefined", "-fno-sanitize-recover=all",
            "-fno-omit-frame-pointer", "-march=x86-64-v3", "-D__HIP_PLATFORM_AMD__",
            "-I" + os.path.join(ROOT, "include"), "-I" + os.path.join(ROOT, "include", "mini-gaussian-splatting"), "-I" + hip_include,
            "-I" + NATIVE,

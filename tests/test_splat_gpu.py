@@ -278,3 +278,137 @@ def test_full_size_config5_properties(gpu):
     assert torch.equal(image, image2)
     ctx.close()
     ctx2.close()
+
+
+# ---- the tile lists themselves (integer work: must equal what the oracle's rectangles and the depths imply) ----
+
+def _expected_lists(rects, depth, tiles_x, tiles_y):
+    """Per tile (row-major), the Gaussians whose rectangle covers it, by (depth, index)."""
+    rc = rects.astype(np.int64)
+    nx = np.maximum(0, rc[:, 2] - rc[:, 0] + 1)
+    ny = np.maximum(0, rc[:, 3] - rc[:, 1] + 1)
+    count = nx * ny
+    g = np.repeat(np.arange(rc.shape[0]), count)
+    local = np.arange(count.sum()) - np.repeat(np.cumsum(count) - count, count)
+    tile = (rc[g, 1] + local // np.maximum(nx[g], 1)) * tiles_x + rc[g, 0] + local % np.maximum(nx[g], 1)
+    order = np.lexsort((g, depth[g], tile))
+    tile, g = tile[order], g[order]
+    begin = np.searchsorted(tile, np.arange(tiles_x * tiles_y), side="left")
+    end = np.searchsorted(tile, np.arange(tiles_x * tiles_y), side="right")
+    return begin, end, g
+
+
+def _assert_lists(ctx, oracle, W, H, params, depth):
+    ref = oracle.splat_step(W, H, params, depth, np.zeros((H, W, 3), np.float32), np.float32, want_grads=False)
+    tiles_x, tiles_y = (W + 15) // 16, (H + 15) // 16
+    want_begin, want_end, want_ids = _expected_lists(ref["rects"], depth, tiles_x, tiles_y)
+    begin, end, ids = ctx.lists()
+    assert ids.size == want_ids.size == ref["pairs"]
+    assert np.array_equal(end - begin, want_end - want_begin)  # every tile's length
+    # the lists may sit anywhere in the array; tile by tile their contents must be equal, in order
+    got = np.concatenate([ids[b:e] for b, e in zip(begin, end)]) if ids.size else ids
+    assert np.array_equal(got, want_ids.astype(np.uint32))
+    # and they tile the array exactly once
+    covered = np.zeros(ids.size + 1, np.int64)
+    np.add.at(covered, begin, 1)
+    np.add.at(covered, end, -1)
+    assert np.all(np.cumsum(covered)[:-1] == 1)
+
+
+@pytest.mark.parametrize("G,W,H,scale", [
+    (1, 16, 16, (2.0, 4.0)),
+    (50, 33, 17, (1.0, 6.0)),        # one supertile, ragged image
+    (700, 130, 260, (1.0, 30.0)),    # several supertiles, the last ones partly outside the image
+    (5000, 640, 400, (0.5, 40.0)),   # rectangles that span many supertiles
+    (20000, 2100, 1100, (1.0, 8.0)), # more than one group of 64 supertiles
+])
+def test_tile_lists_equal_what_rectangles_and_depths_imply(gpu, oracle, G, W, H, scale):
+    import torch
+
+    from xyz_autodiff_cuda_amd import splat
+
+    params, depth = random_scene(G, W, H, seed=G + 3, scale_px=scale)
+    depth[::5] = depth[min(2, G - 1)]  # ties: the index decides
+    if G > 100:
+        params[0, :3] = -1e4   # off screen: no pairs
+        params[2:4, 3] = np.log(5000.0)  # one Gaussian over the whole image
+    ctx = splat.SplatContext(W, H, G)
+    ctx.forward(torch.from_numpy(params).to(gpu), torch.from_numpy(depth).to(gpu))
+    _assert_lists(ctx, oracle, W, H, params, depth)
+    ctx.close()
+
+
+@pytest.mark.parametrize("mode", ["static", "every_step"])
+def test_steps_that_do_not_wait(gpu, oracle, mode):
+    """Without a loss read-back a step only queues work; results equal those of the default mode."""
+    import torch
+
+    from xyz_autodiff_cuda_amd import splat
+
+    G, W, H = 900, 160, 112
+    params, depth = random_scene(G, W, H, seed=31, scale_px=(1.0, 14.0))
+    target = np.random.default_rng(4).uniform(0, 1, (H, W, 3)).astype(np.float32)
+    p, t = torch.from_numpy(params).to(gpu), torch.from_numpy(target).to(gpu)
+    ctx = splat.SplatContext(W, H, G, depth_mode=mode)
+    depths = [depth, depth, (1.0 - depth).astype(np.float32)] if mode == "every_step" else [depth, depth, depth]
+    for d in depths:
+        image, grads, loss = ctx.step(p, torch.from_numpy(d).to(gpu), t, want_loss=False)
+        assert loss is None
+        torch.cuda.synchronize()
+        ref = oracle.splat_step(W, H, params, d, target, np.float32)
+        assert np.abs(image.cpu().numpy() - ref["image"]).max() < 1e-5
+        scale = np.abs(ref["grads"]).max(axis=0) + 1e-20
+        assert (np.abs(grads.cpu().numpy() - ref["grads"]) / scale).max() < 5e-3
+        assert ctx.stats()["pairs"] == ref["pairs"]
+    ctx.close()
+
+
+def test_static_mode_reports_a_changed_depth(gpu, xad):
+    import torch
+
+    from xyz_autodiff_cuda_amd import splat
+
+    G, W, H = 300, 96, 96
+    params, depth = random_scene(G, W, H, seed=12, scale_px=(2.0, 10.0))
+    p, t = torch.from_numpy(params).to(gpu), torch.zeros(H, W, 3, device=gpu)
+    ctx = splat.SplatContext(W, H, G, depth_mode="static")
+    ctx.step(p, torch.from_numpy(depth).to(gpu), t)
+    changed = depth.copy()
+    changed[7] += 0.25
+    ctx.step(p, torch.from_numpy(changed).to(gpu), t, want_loss=False)  # queued; cannot report anything
+    with pytest.raises(xad.XadError, match="XAD_SPLAT_DEPTH_STATIC"):
+        ctx.step(p, torch.from_numpy(changed).to(gpu), t)
+    ctx.step(p, torch.from_numpy(changed).to(gpu), t)  # reordered by the call after the report: fine again
+    ctx.close()
+
+
+def test_overflow_in_a_step_that_does_not_wait_is_reported_later(gpu, oracle, xad):
+    import torch
+
+    from xyz_autodiff_cuda_amd import splat
+
+    G, W, H = 600, 256, 256
+    small, depth = random_scene(G, W, H, seed=5, scale_px=(0.5, 1.0))
+    large = small.copy()
+    large[2:4] += np.log(30.0)  # the same Gaussians, thirty times wider: many times the pairs
+    target = np.zeros((H, W, 3), np.float32)
+    d, t = torch.from_numpy(depth).to(gpu), torch.from_numpy(target).to(gpu)
+    ctx = splat.SplatContext(W, H, G, pair_capacity_hint=4000, depth_mode="static")
+    ctx.step(torch.from_numpy(small).to(gpu), d, t)  # sized for the small scene
+    few = ctx.stats()["pairs"]
+    ctx.step(torch.from_numpy(large).to(gpu), d, t, want_loss=False)  # does not fit, and nobody is told yet
+    with pytest.raises(xad.XadError, match="incomplete"):
+        ctx.step(torch.from_numpy(small).to(gpu), d, t)
+    image, grads, loss = ctx.step(torch.from_numpy(large).to(gpu), d, t)  # the lists were enlarged: complete now
+    ref = oracle.splat_step(W, H, large, depth, target, np.float32)
+    assert ctx.stats()["pairs"] == ref["pairs"] > 4 * few
+    # (every pixel composites hundreds of these wide Gaussians: a few 1e-5 of fp32 rounding; what is being
+    # checked is that no pair is missing, which would show as an error of the size of an alpha)
+    assert np.abs(image.cpu().numpy() - ref["image"]).max() < 5e-5
+    # a step that reads the loss and does not fit is simply run again with larger lists
+    ctx2 = splat.SplatContext(W, H, G, pair_capacity_hint=4000, depth_mode="static")
+    ctx2.step(torch.from_numpy(small).to(gpu), d, t)
+    image2, _, loss2 = ctx2.step(torch.from_numpy(large).to(gpu), d, t)
+    assert np.abs(image2.cpu().numpy() - ref["image"]).max() < 5e-5 and abs(loss2 - ref["loss"]) <= 1e-5 * ref["loss"] + 1e-9
+    ctx.close()
+    ctx2.close()

@@ -60,7 +60,9 @@ __global__ void __launch_bounds__(kSingleBlock) chain_single_kernel(ChainBuffers
 }
 
 // One lane, four consecutive problems, 16-byte accesses (1 KiB per wavefront instruction).  `groups` = n / 4.
-inline __global__ void __launch_bounds__(kQuadBlock) chain_quad_kernel(ChainBuffers buf, std::size_t groups) {
+// (A template, like the copy below, so that only a translation unit that launches it carries its code.)
+template <int kUnused = 0>
+__global__ void __launch_bounds__(kQuadBlock) chain_quad_kernel(ChainBuffers buf, std::size_t groups) {
     using namespace xyz_autodiff::soa;
     const std::size_t g = static_cast<std::size_t>(blockIdx.x) * kQuadBlock + threadIdx.x;
     if (g >= groups) return;
@@ -87,8 +89,9 @@ inline __global__ void __launch_bounds__(kQuadBlock) chain_quad_kernel(ChainBuff
 
 // Plain copy with the chain kernel's access pattern (4 bytes per lane, non-temporal):
 // the yardstick that hardware counters and achievable bandwidth are scaled by.
-inline __global__ void __launch_bounds__(kSingleBlock) stream_copy_kernel(const float* __restrict__ src,
-                                                                          float* __restrict__ dst, std::size_t n) {
+template <int kUnused = 0>
+__global__ void __launch_bounds__(kSingleBlock) stream_copy_kernel(const float* __restrict__ src, float* __restrict__ dst,
+                                                                   std::size_t n) {
     const std::size_t i = static_cast<std::size_t>(blockIdx.x) * kSingleBlock + threadIdx.x;
     if (i < n) __builtin_nontemporal_store(__builtin_nontemporal_load(src + i), dst + i);
 }

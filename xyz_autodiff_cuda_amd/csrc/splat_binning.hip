@@ -1,0 +1,459 @@
+// Binning of the splatting step: from the tile rectangle of every Gaussian to one list of Gaussians
+// per tile, each in (depth, index) order.  Integer work only; no library primitive, no host read-back.
+//
+// The lists are a sparse transpose: Gaussian-major (a rectangle of tiles per Gaussian) to tile-major.
+// A comparison sort or a radix sort of (tile, Gaussian) pairs moves every pair several times; here a
+// pair is written once.  The Gaussians are walked in depth order, and what keeps each list in that
+// order is the walk itself, not a sort:
+//
+//   level A   Gaussians -> supertiles (8 x 8 tiles).  A wavefront takes a range of the depth-ordered
+//             Gaussians and 64 supertiles, one per lane.  64 Gaussians are loaded at a time, one per
+//             lane; the rectangle of each in turn is broadcast (v_readlane) and every lane tests its
+//             own supertile against it.  A first pass counts, the counts of all (supertile, range)
+//             cells are scanned in supertile-major order, and a second pass writes each Gaussian at
+//             its lane's cursor.  Ranges are visited in order inside every supertile, Gaussians in
+//             order inside every range: the list of a supertile comes out in depth order.
+//   level B   supertile -> its 64 tiles: a wavefront takes 64 entries of one supertile's list, one per
+//             lane.  The lane that loads a Gaussian forms the 64-bit mask of the tiles its rectangle
+//             covers inside the supertile (row mask x column multiplier).  Those 64 masks are a 64 x 64
+//             bit matrix, entries by tiles; it is transposed across the lanes in six exchange steps,
+//             after which lane t holds, for tile t, the mask of the entries that cover it: its
+//             population count is the tile's count, and its set bits, walked from the lowest, are the
+//             tile's Gaussians in list order.
+//
+// Work per (Gaussian, supertile) pair is a handful of wavefront instructions; the stores of the final
+// lists are 4 bytes per pair, each pair once.  All sizes that depend on the data (pairs per
+// supertile, pairs in total) stay on the device: grids are sized by the capacity of the buffers, idle
+// wavefronts leave at once, every store is checked against the capacity, and an overflow is
+// recorded in the status words for the host to see whenever it next waits for the stream.
+//
+// Replaces, for the tile-binned renderer, what the reference does not have at all: its renderer
+// visits every Gaussian at every pixel (examples/mini-gaussian-splatting/gaussian_splatting_kernel.cu:33-62).
+#include <xyz_autodiff/accumulate.cuh>
+
+#include "common.cuh"
+#include "splat.cuh"
+#include "splat_launch.cuh"
+
+namespace xad_splat {
+
+namespace {
+
+using xyz_autodiff::accumulate::wave::ballot;
+
+__device__ __forceinline__ std::uint32_t read_lane(std::uint32_t v, int lane) {
+    return static_cast<std::uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(v), lane));
+}
+
+// ---------------------------------------------------------------------------
+// Exclusive scan of n 32-bit counts, in place, in one launch (chained scan with decoupled look-back).
+// Blocks take tickets, so a block only ever waits for blocks that are already running.  The state
+// words carry the launch's epoch, so nothing has to be cleared between launches: a word of another
+// epoch simply is not there yet.  data[n] receives the total.
+constexpr unsigned kScanBlock = 256;
+constexpr unsigned kScanItems = 8;
+constexpr unsigned kScanTile = kScanBlock * kScanItems;
+
+__device__ __forceinline__ std::uint64_t scan_word(std::uint32_t epoch, std::uint32_t inclusive, std::uint32_t value) {
+    return (static_cast<std::uint64_t>((epoch << 1) | inclusive) << 32) | value;
+}
+
+__global__ void __launch_bounds__(kScanBlock) scan_kernel(std::uint32_t* __restrict__ data, std::uint32_t n,
+                                                          std::uint64_t* __restrict__ state, std::uint32_t* __restrict__ tickets,
+                                                          std::uint32_t ticket_base, std::uint32_t epoch) {
+    __shared__ std::uint32_t shared[kScanBlock];
+    __shared__ std::uint32_t block_index, block_exclusive;
+    const unsigned t = threadIdx.x;
+    if (t == 0) block_index = atomicAdd(tickets, 1u) - ticket_base;
+    __syncthreads();
+    const std::uint32_t b = block_index;
+    const std::uint32_t first = b * kScanTile + t * kScanItems;
+
+    std::uint32_t v[kScanItems];
+    if (first + kScanItems <= n) {
+        const uint4 lo = *reinterpret_cast<const uint4*>(data + first), hi = *reinterpret_cast<const uint4*>(data + first + 4);
+        v[0] = lo.x; v[1] = lo.y; v[2] = lo.z; v[3] = lo.w;
+        v[4] = hi.x; v[5] = hi.y; v[6] = hi.z; v[7] = hi.w;
+    } else {
+#pragma unroll
+        for (unsigned k = 0; k < kScanItems; ++k) v[k] = first + k < n ? data[first + k] : 0u;
+    }
+    std::uint32_t mine = 0;
+#pragma unroll
+    for (unsigned k = 0; k < kScanItems; ++k) mine += v[k];
+
+    // inclusive scan of the 256 per-thread sums through LDS
+    shared[t] = mine;
+    __syncthreads();
+    for (unsigned step = 1; step < kScanBlock; step *= 2) {
+        const std::uint32_t other = t >= step ? shared[t - step] : 0u;
+        __syncthreads();
+        shared[t] += other;
+        __syncthreads();
+    }
+    const std::uint32_t thread_exclusive = shared[t] - mine;
+    const std::uint32_t aggregate = shared[kScanBlock - 1];
+
+    // Look-back, by the block's first wavefront: 64 predecessors at a time, nearest first.  Each lane waits
+    // for its predecessor's word of this epoch (that block holds an earlier ticket, so it is running),
+    // the sums up to and including the nearest inclusive prefix are added, and if there was none among
+    // the 64 the next 64 are looked at.  Lanes that would reach before block 0 count as an inclusive zero.
+    if (t < 64) {
+        if (b > 0 && t == 0) __hip_atomic_store(state + b, scan_word(epoch, 0u, aggregate), __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+        std::uint32_t exclusive = 0;
+        for (std::int64_t nearest = static_cast<std::int64_t>(b) - 1; nearest >= 0; nearest -= 64) {
+            const std::int64_t mine_at = nearest - static_cast<std::int64_t>(t);
+            std::uint64_t word = scan_word(epoch, 1u, 0u);
+            if (mine_at >= 0) {
+                do {
+                    word = __hip_atomic_load(state + mine_at, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT);
+                } while (static_cast<std::uint32_t>(word >> 33) != epoch);
+            }
+            const std::uint64_t inclusive = ballot(((word >> 32) & 1u) != 0);
+            const unsigned stop = static_cast<unsigned>(__builtin_ctzll(inclusive | (std::uint64_t(1) << 63)));
+            std::uint32_t part = t <= stop ? static_cast<std::uint32_t>(word) : 0u;
+            for (int offset = 32; offset > 0; offset >>= 1) part += __shfl_xor(part, offset, 64);
+            exclusive += part;
+            if (inclusive != 0) break;
+        }
+        if (t == 0) {
+            __hip_atomic_store(state + b, scan_word(epoch, 1u, exclusive + aggregate), __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+            block_exclusive = exclusive;
+            if (static_cast<std::uint64_t>(b + 1) * kScanTile >= n) data[n] = exclusive + aggregate;  // the last block: the total
+        }
+    }
+    __syncthreads();
+
+    std::uint32_t running = block_exclusive + thread_exclusive;
+    if (first + kScanItems <= n) {
+        std::uint32_t out[kScanItems];
+#pragma unroll
+        for (unsigned k = 0; k < kScanItems; ++k) {
+            out[k] = running;
+            running += v[k];
+        }
+        *reinterpret_cast<uint4*>(data + first) = uint4{out[0], out[1], out[2], out[3]};
+        *reinterpret_cast<uint4*>(data + first + 4) = uint4{out[4], out[5], out[6], out[7]};
+    } else {
+#pragma unroll
+        for (unsigned k = 0; k < kScanItems; ++k) {
+            if (first + k < n) data[first + k] = running;
+            running += v[k];
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Level A.  One wavefront per block; block = (range of Gaussians) x (group of 64 supertiles), blocks of
+// one range adjacent so that they read the same rectangles from the same L2.
+// kFill = false: matrix_a[supertile * ranges_a + range] = number of Gaussians of the range that
+// touch the supertile.  kFill = true: matrix_a holds the scanned counts; the Gaussians are written.
+// rects_by_depth[i] is the rectangle of Gaussian by_depth[i]: both loads of a lane are independent and coalesced.
+template <bool kFill>
+__global__ void __launch_bounds__(64) super_kernel(BinPlan p, const std::uint32_t* __restrict__ by_depth,
+                                                   const TileRect* __restrict__ rects_by_depth,
+                                                   std::uint32_t* __restrict__ matrix_a, std::uint32_t* __restrict__ list_a) {
+    const int lane = static_cast<int>(threadIdx.x);
+    const int group = static_cast<int>(blockIdx.x % static_cast<unsigned>(p.groups));
+    const int range = static_cast<int>(blockIdx.x / static_cast<unsigned>(p.groups));
+    const int s = group * 64 + lane;
+    const bool owner = s < p.supers;
+    const int sx = s % p.super_x, sy = s / p.super_x;
+    // rows of supertiles this group reaches into
+    const int last_super = group * 64 + 63 < p.supers - 1 ? group * 64 + 63 : p.supers - 1;
+    const int row_lo = (group * 64) / p.super_x, row_hi = last_super / p.super_x;
+    const std::size_t cell = static_cast<std::size_t>(owner ? s : 0) * p.ranges_a + range;
+    std::uint32_t cursor = (kFill && owner) ? matrix_a[cell] : 0u;
+    std::uint32_t count = 0;
+
+    const int first = range * p.range_a;
+    const int last = first + p.range_a < p.G ? first + p.range_a : p.G;
+    for (int base = first; base < last; base += 64) {
+        const int i = base + lane;
+        std::uint32_t g = 0, lo = 0, hi = 0;
+        bool candidate = false;
+        if (i < last) {
+            g = by_depth[i];
+            const TileRect rc = rects_by_depth[i];
+            if (rc.x0 <= rc.x1) {
+                const int y0 = rc.y0 >> 3, y1 = rc.y1 >> 3;
+                candidate = y1 >= row_lo && y0 <= row_hi;
+                lo = static_cast<std::uint32_t>(rc.x0 >> 3) | (static_cast<std::uint32_t>(y0) << 16);
+                hi = static_cast<std::uint32_t>(rc.x1 >> 3) | (static_cast<std::uint32_t>(y1) << 16);
+            }
+        }
+        for (std::uint64_t todo = ballot(candidate); todo != 0; todo &= todo - 1) {
+            const int j = __builtin_ctzll(todo);
+            const std::uint32_t l = read_lane(lo, j), h = read_lane(hi, j), gj = read_lane(g, j);
+            const int x0 = static_cast<int>(l & 0xffffu), y0 = static_cast<int>(l >> 16);
+            const int x1 = static_cast<int>(h & 0xffffu), y1 = static_cast<int>(h >> 16);
+            const bool covered = owner && sx >= x0 && sx <= x1 && sy >= y0 && sy <= y1;
+            if constexpr (kFill) {
+                if (covered) {
+                    if (cursor < p.capacity_a) list_a[cursor] = gj;
+                    ++cursor;
+                }
+            } else {
+                count += covered ? 1u : 0u;
+            }
+        }
+    }
+    if constexpr (!kFill) {
+        if (owner) matrix_a[cell] = count;
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Between the levels: how many wavefronts every supertile's list needs at level B (at least one, so
+// that every tile gets its range written), as a prefix over the supertiles, clamped to the grid that
+// will be launched.  One block.  Also records the number of (supertile, Gaussian) pairs and whether
+// they fit, and clears the tile ranges (tiles that no wavefront reaches keep an empty range).
+__global__ void __launch_bounds__(256) plan_kernel(BinPlan p, const std::uint32_t* __restrict__ offsets_a,
+                                                   std::uint32_t* __restrict__ first_wave, std::uint32_t* __restrict__ tile_ranges,
+                                                   std::uint32_t* __restrict__ status, bool clear_depth_flag) {
+    __shared__ std::uint32_t shared[256];
+    __shared__ std::uint32_t carried;
+    const unsigned t = threadIdx.x;
+    for (std::size_t k = static_cast<std::size_t>(blockIdx.x) * 256 + t; k < static_cast<std::size_t>(p.tiles_x) * p.tiles_y * 2;
+         k += static_cast<std::size_t>(gridDim.x) * 256)
+        tile_ranges[k] = 0;
+    if (blockIdx.x != 0) return;
+    if (t == 0) carried = 0;
+    __syncthreads();
+    for (int base = 0; base < p.supers; base += 256) {
+        const int s = base + static_cast<int>(t);
+        std::uint32_t waves = 0;
+        if (s < p.supers) {
+            std::uint32_t begin = offsets_a[static_cast<std::size_t>(s) * p.ranges_a];
+            std::uint32_t end = offsets_a[static_cast<std::size_t>(s + 1) * p.ranges_a];
+            begin = begin < p.capacity_a ? begin : p.capacity_a;
+            end = end < p.capacity_a ? end : p.capacity_a;
+            waves = (end - begin + kBinRangeB - 1) / kBinRangeB;
+            if (waves == 0) waves = 1;
+        }
+        shared[t] = waves;
+        __syncthreads();
+        for (unsigned step = 1; step < 256; step *= 2) {
+            const std::uint32_t other = t >= step ? shared[t - step] : 0u;
+            __syncthreads();
+            shared[t] += other;
+            __syncthreads();
+        }
+        const std::uint32_t exclusive = carried + shared[t] - waves;
+        if (s < p.supers) first_wave[s] = exclusive < p.waves_b ? exclusive : p.waves_b;
+        __syncthreads();
+        if (t == 255) carried += shared[255];
+        __syncthreads();
+    }
+    if (t == 0) {
+        first_wave[p.supers] = carried < p.waves_b ? carried : p.waves_b;
+        const std::uint32_t super_pairs = offsets_a[static_cast<std::size_t>(p.supers) * p.ranges_a];
+        status[kStatusSuperPairs] = super_pairs;
+        // this step's verdict starts here; the last kernel of the binning may still raise it
+        const bool overflow = super_pairs > p.capacity_a || carried > p.waves_b;
+        status[kStatusOverflow] = overflow ? 1u : 0u;
+        if (overflow) atomicMax(status + kStatusOverflowSticky, super_pairs > p.capacity ? super_pairs : p.capacity + 1);
+        if (clear_depth_flag) status[kStatusDepthChanged] = 0;  // the projection of this step has set it, the host has its copy
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Transpose of a 64 x 64 bit matrix held one row per lane (lo = columns 0..31, hi = columns 32..63):
+// afterwards lane t holds column t, bit j of it being bit t of lane j's row.  The usual recursive block
+// swap: at distance k, the lanes whose bit k is clear keep their columns with bit k clear and receive,
+// into their columns with bit k set, the partner's columns with bit k clear; the others the reverse.
+__device__ __forceinline__ void transpose_64x64(std::uint32_t& lo, std::uint32_t& hi, int lane) {
+    {
+        const std::uint32_t other_lo = __shfl_xor(lo, 32, 64), other_hi = __shfl_xor(hi, 32, 64);
+        if (lane & 32)
+            lo = other_hi;
+        else
+            hi = other_lo;
+    }
+    constexpr std::uint32_t kClear[5] = {0x0000ffffu, 0x00ff00ffu, 0x0f0f0f0fu, 0x33333333u, 0x55555555u};
+#pragma unroll
+    for (int step = 0; step < 5; ++step) {
+        const int k = 16 >> step;
+        const std::uint32_t m = kClear[step];
+        const std::uint32_t other_lo = __shfl_xor(lo, k, 64), other_hi = __shfl_xor(hi, k, 64);
+        if (lane & k) {
+            lo = ((other_lo >> k) & m) | (lo & ~m);
+            hi = ((other_hi >> k) & m) | (hi & ~m);
+        } else {
+            lo = (lo & m) | ((other_lo & m) << k);
+            hi = (hi & m) | ((other_hi & m) << k);
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Level B.  One wavefront per block: wavefront w serves entries [64 q, 64 q + 64) of the list of supertile s,
+// where first_wave[s] <= w < first_wave[s + 1] and q = w - first_wave[s]; after the transpose, lane = tile of
+// the supertile (row-major, 8 per row).  The counts of supertile s live at
+// matrix_b[64 first_wave[s] + tile * waves_of_s + q]: scanned as one flat array, that order puts every
+// tile's pieces next to each other and the tiles of a supertile one after the other, so the scanned
+// value is the position in the final list.  Wavefronts beyond the last supertile clear their 64 cells
+// and leave.
+template <bool kFill>
+__global__ void __launch_bounds__(64) tile_kernel(BinPlan p, const std::uint32_t* __restrict__ offsets_a,
+                                                  const std::uint32_t* __restrict__ first_wave,
+                                                  const std::uint32_t* __restrict__ list_a, const TileRect* __restrict__ rects,
+                                                  std::uint32_t* __restrict__ matrix_b, std::uint32_t* __restrict__ list,
+                                                  std::uint32_t* __restrict__ range_begin, std::uint32_t* __restrict__ range_end,
+                                                  std::uint32_t* __restrict__ status) {
+    const int lane = static_cast<int>(threadIdx.x);
+    const std::uint32_t w = blockIdx.x;
+    const std::uint32_t used = first_wave[p.supers];
+    if (w >= used) {
+        if constexpr (!kFill) matrix_b[static_cast<std::size_t>(w) * 64 + lane] = 0;
+        return;
+    }
+    // the last supertile whose first wavefront is not after w
+    int s = 0;
+    for (int hi = p.supers; hi - s > 1;) {
+        const int mid = (s + hi) / 2;
+        if (first_wave[mid] <= w)
+            s = mid;
+        else
+            hi = mid;
+    }
+    const std::uint32_t wave0 = first_wave[s], waves = first_wave[s + 1] - wave0, q = w - wave0;
+    std::uint32_t begin = offsets_a[static_cast<std::size_t>(s) * p.ranges_a];
+    std::uint32_t end = offsets_a[static_cast<std::size_t>(s + 1) * p.ranges_a];
+    begin = begin < p.capacity_a ? begin : p.capacity_a;
+    end = end < p.capacity_a ? end : p.capacity_a;
+    const std::uint32_t i = begin + q * kBinRangeB + static_cast<std::uint32_t>(lane);
+
+    const int base_x = (s % p.super_x) * 8, base_y = (s / p.super_x) * 8;
+    std::uint32_t g = 0, mask_lo = 0, mask_hi = 0;
+    if (i < end) {
+        g = list_a[i];
+        const TileRect rc = rects[g];
+        const int x0 = rc.x0 - base_x > 0 ? rc.x0 - base_x : 0, x1 = rc.x1 - base_x < 7 ? rc.x1 - base_x : 7;
+        const int y0 = rc.y0 - base_y > 0 ? rc.y0 - base_y : 0, y1 = rc.y1 - base_y < 7 ? rc.y1 - base_y : 7;
+        if (x0 <= x1 && y0 <= y1) {
+            // bits x0..x1 of a row, repeated in rows y0..y1 (the multiplier has one bit per row: no carries)
+            const std::uint64_t row = ((std::uint64_t(1) << (x1 - x0 + 1)) - 1) << x0;
+            const std::uint64_t rows = (0x0101010101010101ull >> (8 * (7 - (y1 - y0)))) << (8 * y0);
+            const std::uint64_t mask = row * rows;
+            mask_lo = static_cast<std::uint32_t>(mask);
+            mask_hi = static_cast<std::uint32_t>(mask >> 32);
+        }
+    }
+    transpose_64x64(mask_lo, mask_hi, lane);  // now: which of the 64 entries cover this lane's tile
+    const int tx = base_x + (lane & 7), ty = base_y + (lane >> 3);
+    const bool owner = tx < p.tiles_x && ty < p.tiles_y;
+    std::uint64_t mine = owner ? (static_cast<std::uint64_t>(mask_hi) << 32) | mask_lo : 0;
+    const std::size_t cell = static_cast<std::size_t>(wave0) * 64 + static_cast<std::size_t>(lane) * waves + q;
+
+    if constexpr (!kFill) {
+        matrix_b[cell] = static_cast<std::uint32_t>(__builtin_popcountll(mine));
+    } else {
+        std::uint32_t cursor = matrix_b[cell];
+        const std::uint32_t from = cursor;
+        // every lane stays in the loop until the last one is done: the exchange below reads other lanes' registers
+        while (ballot(mine != 0) != 0) {
+            const bool has = mine != 0;
+            const int j = has ? __builtin_ctzll(mine) : 0;
+            const std::uint32_t gj = __shfl(g, j, 64);
+            if (has) {
+                if (cursor < p.capacity) list[cursor] = gj;
+                ++cursor;
+                mine &= mine - 1;
+            }
+        }
+        if (q == 0 && owner) {
+            // this tile's list: from the first cell of the tile to the first cell of the next one
+            const std::size_t next_cell = static_cast<std::size_t>(wave0) * 64 + static_cast<std::size_t>(lane + 1) * waves;
+            const std::uint32_t to = matrix_b[next_cell];
+            const int tile = ty * p.tiles_x + tx;
+            range_begin[tile] = from < p.capacity ? from : p.capacity;
+            range_end[tile] = to < p.capacity ? to : p.capacity;
+        }
+        if (w == 0 && lane == 0) {
+            const std::uint32_t pairs = matrix_b[static_cast<std::size_t>(p.waves_b) * 64];  // the scan's total
+            status[kStatusPairs] = pairs;
+            if (pairs > p.capacity) {
+                status[kStatusOverflow] = 1;
+                atomicMax(status + kStatusOverflowSticky, pairs);
+            }
+        }
+    }
+}
+
+}  // namespace
+
+BinPlan make_bin_plan(int G, int tiles_x, int tiles_y, std::uint32_t capacity, std::uint32_t capacity_a) {
+    BinPlan p{};
+    p.G = G;
+    p.tiles_x = tiles_x;
+    p.tiles_y = tiles_y;
+    p.super_x = (tiles_x + 7) / 8;
+    p.super_y = (tiles_y + 7) / 8;
+    p.supers = p.super_x * p.super_y;
+    p.groups = (p.supers + 63) / 64;
+    // about 8192 wavefronts at level A (short ones: a wavefront's chunks of 64 Gaussians are a chain of memory
+    // latencies), and never less than 64 Gaussians per wavefront
+    const long long per_wave = (static_cast<long long>(G) * p.groups + 8191) / 8192;
+    p.range_a = static_cast<int>(((per_wave > 64 ? per_wave : 64) + 63) / 64 * 64);
+    p.ranges_a = (G + p.range_a - 1) / p.range_a;
+    p.capacity = capacity;
+    p.capacity_a = capacity_a < capacity ? capacity_a : capacity;
+    p.waves_b = static_cast<std::uint32_t>((static_cast<std::uint64_t>(p.capacity_a) + kBinRangeB - 1) / kBinRangeB) +
+                static_cast<std::uint32_t>(p.supers);
+    return p;
+}
+
+std::size_t bin_matrix_a_words(const BinPlan& p) { return static_cast<std::size_t>(p.supers) * p.ranges_a + 1; }
+std::size_t bin_matrix_b_words(const BinPlan& p) { return static_cast<std::size_t>(p.waves_b) * 64 + 1; }
+std::size_t bin_scan_state_words(const BinPlan& p) {
+    const std::size_t longest = bin_matrix_a_words(p) > bin_matrix_b_words(p) ? bin_matrix_a_words(p) : bin_matrix_b_words(p);
+    return (longest + kScanTile - 1) / kScanTile + 1;
+}
+
+namespace {
+
+int launch_scan(hipStream_t s, std::uint32_t* data, std::size_t n, BinScratch& scratch) {
+    XAD_REQUIRE(n > 0 && n < (std::size_t(1) << 32) - 2 * kScanTile, "splat binning: %zu counts do not fit the 32-bit scan", n);
+    const unsigned blocks = static_cast<unsigned>((n + kScanTile - 1) / kScanTile);
+    scratch.epoch = (scratch.epoch + 1) & 0x3fffffffu;
+    if (scratch.epoch == 0) scratch.epoch = 1;  // state words start as zero: epoch 0 is never used
+    hipLaunchKernelGGL(scan_kernel, dim3(blocks), dim3(kScanBlock), 0, s, data, static_cast<std::uint32_t>(n), scratch.scan_state,
+                       scratch.tickets, scratch.tickets_taken, scratch.epoch);
+    XAD_HIP_TRY(hipGetLastError());
+    scratch.tickets_taken += blocks;  // wraps like the device counter
+    return XAD_OK;
+}
+
+}  // namespace
+
+int launch_binning(hipStream_t s, const BinPlan& p, const std::uint32_t* by_depth, const TileRect* rects_by_depth,
+                   const TileRect* rects, BinScratch& scratch,
+                   std::uint32_t* list, std::uint32_t* range_begin, std::uint32_t* range_end, std::uint32_t* status,
+                   bool clear_depth_flag) {
+    XAD_REQUIRE(p.G > 0 && p.supers > 0 && p.ranges_a > 0 && p.capacity > 0, "splat binning: empty plan");
+    XAD_REQUIRE(range_end == range_begin + static_cast<std::size_t>(p.tiles_x) * p.tiles_y,
+                "splat binning: the two halves of the tile ranges must be adjacent");
+    const unsigned waves_a = static_cast<unsigned>(p.ranges_a) * static_cast<unsigned>(p.groups);
+    hipLaunchKernelGGL(super_kernel<false>, dim3(waves_a), dim3(64), 0, s, p, by_depth, rects_by_depth, scratch.matrix_a,
+                       scratch.list_a);
+    XAD_HIP_TRY(hipGetLastError());
+    if (int st = launch_scan(s, scratch.matrix_a, bin_matrix_a_words(p) - 1, scratch)) return st;
+    const unsigned plan_blocks = static_cast<unsigned>((static_cast<std::size_t>(p.tiles_x) * p.tiles_y * 2 + 4095) / 4096);
+    hipLaunchKernelGGL(plan_kernel, dim3(plan_blocks < 1 ? 1 : (plan_blocks > 512 ? 512 : plan_blocks)), dim3(256), 0, s, p,
+                       scratch.matrix_a, scratch.first_wave, range_begin, status, clear_depth_flag);
+    XAD_HIP_TRY(hipGetLastError());
+    hipLaunchKernelGGL(super_kernel<true>, dim3(waves_a), dim3(64), 0, s, p, by_depth, rects_by_depth, scratch.matrix_a,
+                       scratch.list_a);
+    XAD_HIP_TRY(hipGetLastError());
+    hipLaunchKernelGGL(tile_kernel<false>, dim3(p.waves_b), dim3(64), 0, s, p, scratch.matrix_a, scratch.first_wave, scratch.list_a,
+                       rects, scratch.matrix_b, list, range_begin, range_end, status);
+    XAD_HIP_TRY(hipGetLastError());
+    if (int st = launch_scan(s, scratch.matrix_b, bin_matrix_b_words(p) - 1, scratch)) return st;
+    hipLaunchKernelGGL(tile_kernel<true>, dim3(p.waves_b), dim3(64), 0, s, p, scratch.matrix_a, scratch.first_wave, scratch.list_a,
+                       rects, scratch.matrix_b, list, range_begin, range_end, status);
+    XAD_HIP_TRY(hipGetLastError());
+    return XAD_OK;
+}
+
+}  // namespace xad_splat

@@ -1,5 +1,5 @@
-// The splatting step behind the C ABI: workspace ownership and stage order.
-#include <chrono>
+// The splatting step behind the C ABI: workspace ownership, stage order, and the few places
+// where the host has to look at what the device found.
 #include <new>
 
 #include "common.cuh"
@@ -7,72 +7,131 @@
 
 using namespace xad_splat;
 
+namespace {
+
+// What the device reports back, in pinned host memory: the status words of the step and the loss.
+struct HostReport {
+    std::uint32_t status[kStatusWords];
+    double loss;
+};
+
+__global__ void clear_words_kernel(std::uint32_t* words, int first, int count) {
+    if (static_cast<int>(threadIdx.x) < count) words[first + threadIdx.x] = 0;
+}
+
+}  // namespace
+
 struct xad_splat_context {
     int width = 0, height = 0, G = 0;
     int device = 0;  // the device that was current at creation: owns every buffer below
     int tiles_x = 0, tiles_y = 0, tiles = 0;
-    int key_bits = 0;        // bits of a tile index: what the pair sort looks at
-    bool wide_keys = false;  // more than 65 536 tiles: 32-bit pair keys instead of 16-bit
-    std::uint32_t capacity = 0;  // pairs the workspace can hold
-    std::uint32_t pairs = 0;     // pairs of the last step
+    int depth_mode = XAD_SPLAT_DEPTH_CHECKED;
     bool profile = false;
+    bool order_valid = false;   // by_depth is the (depth, index) order of ordered_depth
+    bool capacity_seen = false;  // a step has been seen to fit the pair lists since they were last sized
+    std::uint32_t pairs = 0;     // pairs of the last step the host has a report of
 
+    // one allocation for everything whose size is fixed by (G, image): `fixed` is its base
+    void* fixed = nullptr;
     Record* records = nullptr;
     TileRect* rects = nullptr;
-    std::uint32_t* counts = nullptr;   // G + 1
-    std::uint32_t* offsets = nullptr;  // G + 2: exclusive scan of counts, then the depth-changed flag
+    TileRect* rects_by_depth = nullptr;  // the same rectangles in depth order
+    std::uint32_t* rank = nullptr;       // G: position of every Gaussian in the depth order
     std::uint32_t *depth_keys = nullptr, *depth_keys_sorted = nullptr;  // G each
-    std::uint32_t *identity = nullptr, *by_depth = nullptr;  // G each; by_depth = Gaussians in (depth, index) order
-    float* ordered_depth = nullptr;  // G: the depths by_depth was computed from
-    bool order_valid = false;
-    std::uint32_t* counts_by_depth = nullptr;  // G + 1, the last one stays zero
-    void *keys = nullptr, *keys_sorted = nullptr;  // 2 or 4 bytes per pair
-    std::uint32_t *ids = nullptr, *ids_sorted = nullptr;
-    std::uint32_t *range_begin = nullptr, *range_end = nullptr;
+    std::uint32_t *identity = nullptr, *by_depth = nullptr;             // G each; by_depth = Gaussians in (depth, index) order
+    float* ordered_depth = nullptr;                                     // G: the depths by_depth was computed from
+    std::uint32_t *range_begin = nullptr, *range_end = nullptr;         // tiles each, adjacent
     float* final_T = nullptr;
     std::uint32_t* n_contrib = nullptr;
-    float* record_grads = nullptr;  // G x 9
+    float* record_grads = nullptr;  // G x kRecordGradStride
     double* loss = nullptr;
-    std::uint32_t* host_pairs = nullptr;  // pinned, 2 words: number of pairs, depth-changed flag
-    double* host_loss = nullptr;          // pinned
-    void* scan_temp = nullptr;
-    std::size_t scan_bytes = 0;
+    std::uint32_t* status = nullptr;  // kStatusWords
     void* depth_sort_temp = nullptr;
     std::size_t depth_sort_bytes = 0;
-    void* sort_temp = nullptr;
-    std::size_t sort_bytes = 0;
 
-    static constexpr int kStages = 7;  // project, scan+emit, sort, ranges, render fwd, render bwd, parameter bwd
+    // one allocation for everything sized by the pair capacity: `paired` is its base
+    void* paired = nullptr;
+    std::uint32_t* list = nullptr;  // the tiles' lists
+    BinPlan plan{};
+    BinScratch bin;
+
+    HostReport* report = nullptr;  // pinned
+
+    static constexpr int kStages = 5;  // project, binning, render forward, render backward, parameter backward
     hipEvent_t marks[kStages + 1] = {};
     float stage_ms[kStages] = {};
-    hipEvent_t count_ready = nullptr;  // the read-back of the pair count has arrived
+    hipEvent_t report_ready = nullptr;
 };
 
 namespace {
 
-int free_pair_buffers(xad_splat_context* c) {
-    (void)hipFree(c->keys);
-    (void)hipFree(c->keys_sorted);
-    (void)hipFree(c->ids);
-    (void)hipFree(c->ids_sorted);
-    (void)hipFree(c->sort_temp);
-    c->keys = c->keys_sorted = nullptr;
-    c->ids = c->ids_sorted = nullptr;
-    c->sort_temp = nullptr;
-    return XAD_OK;
+// Carves consecutive 256-byte aligned pieces out of one allocation; first pass (base == nullptr) only adds up.
+struct Carver {
+    char* base;
+    std::size_t used = 0;
+    template <typename T>
+    T* take(std::size_t count) {
+        const std::size_t at = used;
+        used += (count * sizeof(T) + 255) / 256 * 256;
+        return base ? reinterpret_cast<T*>(base + at) : nullptr;
+    }
+};
+
+void carve_fixed(xad_splat_context* c, char* base, std::size_t* bytes) {
+    Carver k{base};
+    const std::size_t G = static_cast<std::size_t>(c->G), pixels = static_cast<std::size_t>(c->width) * c->height;
+    c->records = k.take<Record>(G);
+    c->rects = k.take<TileRect>(G);
+    c->rects_by_depth = k.take<TileRect>(G);
+    c->rank = k.take<std::uint32_t>(G);
+    c->depth_keys = k.take<std::uint32_t>(G);
+    c->depth_keys_sorted = k.take<std::uint32_t>(G);
+    c->identity = k.take<std::uint32_t>(G);
+    c->by_depth = k.take<std::uint32_t>(G);
+    c->ordered_depth = k.take<float>(G);
+    c->range_begin = k.take<std::uint32_t>(static_cast<std::size_t>(c->tiles) * 2);
+    c->range_end = c->range_begin ? c->range_begin + c->tiles : nullptr;
+    c->final_T = k.take<float>(pixels);
+    c->n_contrib = k.take<std::uint32_t>(pixels);
+    c->record_grads = k.take<float>(G * kRecordGradStride);
+    c->loss = k.take<double>(1);
+    c->status = k.take<std::uint32_t>(kStatusWords);
+    c->bin.tickets = k.take<std::uint32_t>(1);
+    c->depth_sort_temp = k.take<char>(c->depth_sort_bytes ? c->depth_sort_bytes : 16);
+    *bytes = k.used;
 }
 
-int allocate_pair_buffers(xad_splat_context* c, std::uint32_t capacity) {
-    free_pair_buffers(c);
-    c->capacity = 0;  // stays zero if an allocation below fails: the next call then tries again
-    const std::size_t key_bytes = c->wide_keys ? 4 : 2;
-    XAD_HIP_TRY(hipMalloc(&c->keys, key_bytes * capacity));
-    XAD_HIP_TRY(hipMalloc(&c->keys_sorted, key_bytes * capacity));
-    XAD_HIP_TRY(hipMalloc(&c->ids, sizeof(std::uint32_t) * capacity));
-    XAD_HIP_TRY(hipMalloc(&c->ids_sorted, sizeof(std::uint32_t) * capacity));
-    c->sort_bytes = sort_temp_bytes(capacity, c->wide_keys);
-    XAD_HIP_TRY(hipMalloc(&c->sort_temp, c->sort_bytes ? c->sort_bytes : 16));
-    c->capacity = capacity;
+void carve_paired(xad_splat_context* c, char* base, std::size_t* bytes) {
+    Carver k{base};
+    c->list = k.take<std::uint32_t>(c->plan.capacity);
+    c->bin.list_a = k.take<std::uint32_t>(c->plan.capacity);
+    c->bin.matrix_a = k.take<std::uint32_t>(bin_matrix_a_words(c->plan));
+    c->bin.matrix_b = k.take<std::uint32_t>(bin_matrix_b_words(c->plan));
+    c->bin.first_wave = k.take<std::uint32_t>(static_cast<std::size_t>(c->plan.supers) + 1);
+    c->bin.scan_state = k.take<std::uint64_t>(bin_scan_state_words(c->plan));
+    *bytes = k.used;
+}
+
+// (Re)allocates the buffers sized by the pair capacity.  Waits for the device first: a step may still be using them.
+int size_pair_buffers(xad_splat_context* c, std::uint32_t capacity) {
+    if (c->paired) {
+        XAD_HIP_TRY(hipDeviceSynchronize());
+        (void)hipFree(c->paired);
+        c->paired = nullptr;
+    }
+    c->capacity_seen = false;
+    c->plan = make_bin_plan(c->G, c->tiles_x, c->tiles_y, capacity, capacity);  // the buffers are sized for this one
+    std::size_t bytes = 0;
+    carve_paired(c, nullptr, &bytes);
+    void* base = nullptr;
+    if (hipMalloc(&base, bytes) != hipSuccess) {
+        c->plan.capacity = 0;  // the next call tries again
+        return xad::fail(XAD_ERR_HIP, "splat: hipMalloc of %zu bytes for %u pairs failed", bytes, capacity);
+    }
+    c->paired = base;
+    carve_paired(c, static_cast<char*>(base), &bytes);
+    // the scan's state words must not look like words of a coming epoch
+    XAD_HIP_TRY(hipMemset(c->bin.scan_state, 0, bin_scan_state_words(c->plan) * sizeof(std::uint64_t)));
     return XAD_OK;
 }
 
@@ -87,68 +146,97 @@ int order_by_depth(xad_splat_context* c, const float* depth, hipStream_t s) {
     if (int st = sort_by_depth(s, c->depth_sort_temp, c->depth_sort_bytes, c->depth_keys, c->depth_keys_sorted, c->identity,
                                c->by_depth, c->G))
         return st;
+    if (int st = launch_depth_rank(s, c->G, c->by_depth, c->rank)) return st;
     XAD_HIP_TRY(hipMemcpyAsync(c->ordered_depth, depth, sizeof(float) * c->G, hipMemcpyDeviceToDevice, s));
     c->order_valid = true;
     return XAD_OK;
 }
 
-int emit(xad_splat_context* c, hipStream_t s) {
-    std::uint32_t* depth_changed = c->offsets + c->G + 1;
-    return launch_emit(s, c->G, c->by_depth, c->rects, c->offsets, c->tiles_x, c->wide_keys, c->keys, c->ids, c->capacity,
-                       c->range_begin, c->tiles * 2, depth_changed);
+int bin_lists(xad_splat_context* c, hipStream_t s, bool clear_depth_flag) {
+    return launch_binning(s, c->plan, c->by_depth, c->rects_by_depth, c->rects, c->bin, c->list, c->range_begin, c->range_end,
+                          c->status, clear_depth_flag);
 }
 
-// Places the pairs (scan of the tile counts in depth order) and emits them.  The number of pairs,
-// which sizes the sort, and the depth-changed flag are read back: the one wait of a step.  The
-// emission is queued before that wait, so it runs while the host is woken: it needs the offsets,
-// not the count, and never writes past the capacity.  (The copy that reads the flag is ahead of
-// the emission, which resets it, in the stream.)
-int place_and_emit(xad_splat_context* c, hipStream_t s) {
-    if (int st = launch_permute_counts(s, c->G, c->by_depth, c->counts, c->counts_by_depth)) return st;
-    if (int st = exclusive_scan_counts(s, c->scan_temp, c->scan_bytes, c->counts_by_depth, c->offsets, c->G)) return st;
-    XAD_HIP_TRY(hipMemcpyAsync(c->host_pairs, c->offsets + c->G, 2 * sizeof(std::uint32_t), hipMemcpyDeviceToHost, s));
-    XAD_HIP_TRY(hipEventRecord(c->count_ready, s));
-    if (int st = emit(c, s)) return st;
-    XAD_HIP_TRY(hipEventSynchronize(c->count_ready));
-    c->pairs = c->host_pairs[0];
+// Queues a copy of the status words (and the loss) to the host and waits for it.
+int fetch_report(xad_splat_context* c, hipStream_t s) {
+    XAD_HIP_TRY(hipMemcpyAsync(c->report->status, c->status, sizeof(std::uint32_t) * kStatusWords, hipMemcpyDeviceToHost, s));
+    XAD_HIP_TRY(hipMemcpyAsync(&c->report->loss, c->loss, sizeof(double), hipMemcpyDeviceToHost, s));
+    XAD_HIP_TRY(hipEventRecord(c->report_ready, s));
+    XAD_HIP_TRY(hipEventSynchronize(c->report_ready));
+    c->pairs = c->report->status[kStatusPairs];
     return XAD_OK;
 }
 
-// project .. tile ranges; leaves the sorted lists in the context
+int clear_status(xad_splat_context* c, hipStream_t s, int first, int count) {
+    hipLaunchKernelGGL(clear_words_kernel, dim3(1), dim3(64), 0, s, c->status, first, count);
+    XAD_HIP_TRY(hipGetLastError());
+    return XAD_OK;
+}
+
+std::uint32_t grown(std::uint32_t pairs) {
+    const std::uint64_t want = static_cast<std::uint64_t>(pairs) + pairs / 4 + 1024;
+    return static_cast<std::uint32_t>(want < 0xfffffff0ull ? want : 0xfffffff0ull);
+}
+
+// Project and bin; leaves the tiles' lists in the context.  Where the host has to look:
+//   - XAD_SPLAT_DEPTH_CHECKED: whether a depth changed, every call (the binning is queued before the
+//     wait and runs during it; if a depth did change, order and binning are redone);
+//   - the first call after the pair lists were sized: whether the pairs fit (if not, the lists are
+//     enlarged and the binning is redone).
+// Otherwise nothing is read back: an overflow or a depth that changed against the caller's promise is
+// left in the sticky status words for the next call that waits anyway.
 int bin(xad_splat_context* c, const float* params, const float* depth, hipStream_t s) {
     int current = -1;
     XAD_HIP_TRY(hipGetDevice(&current));
     XAD_REQUIRE(current == c->device, "splat: the context belongs to device %d, but device %d is current", c->device, current);
+    if (c->plan.capacity == 0)
+        if (int st = size_pair_buffers(c, static_cast<std::uint32_t>(static_cast<std::size_t>(c->G) * 8 + 1024))) return st;
     mark(c, 0, s);
-    const bool had_order = c->order_valid;
+    const bool had_order = c->order_valid && c->depth_mode != XAD_SPLAT_DEPTH_EVERY_STEP;
     if (!had_order)
         if (int st = order_by_depth(c, depth, s)) return st;
-    std::uint32_t* depth_changed = c->offsets + c->G + 1;  // zero at creation, reset by every emission
-    if (int st = launch_project(s, c->G, params, depth, c->ordered_depth, depth_changed, c->width, c->height, c->records,
-                                c->rects, c->counts, c->record_grads, c->loss))
-        return st;
+    auto project = [&]() {
+        return launch_project(s, c->G, params, depth, c->ordered_depth, c->rank, c->status, c->width, c->height, c->records,
+                              c->rects, c->rects_by_depth, c->record_grads, c->loss);
+    };
+    if (int st = project()) return st;
     mark(c, 1, s);
-    // The order of the previous call is used on the assumption that the depths are the same; the
-    // flag read back with the pair count says whether they were, and if not the placement is redone.
-    if (int st = place_and_emit(c, s)) return st;
-    if (had_order && c->host_pairs[1] != 0) {
-        if (int st = order_by_depth(c, depth, s)) return st;
-        if (int st = place_and_emit(c, s)) return st;
+    const bool check_depth = c->depth_mode == XAD_SPLAT_DEPTH_CHECKED && had_order;
+    if (check_depth) {
+        // the order of the previous call is used on the assumption that the depths are the same; the
+        // flag says whether they were.  The copy is ahead of the binning, which clears the flag.
+        XAD_HIP_TRY(hipMemcpyAsync(c->report->status + kStatusDepthChanged, c->status + kStatusDepthChanged, sizeof(std::uint32_t),
+                                   hipMemcpyDeviceToHost, s));
+        XAD_HIP_TRY(hipEventRecord(c->report_ready, s));
     }
-    if (c->pairs > c->capacity) {
-        // the emission above stopped at the old capacity; hipFree waits for it before the buffers go
-        const std::uint64_t want = static_cast<std::uint64_t>(c->pairs) + c->pairs / 4 + 1024;
-        XAD_REQUIRE(want < 0xffffffffull, "splat: %u pairs exceed the 32-bit pair index", c->pairs);
-        if (int st = allocate_pair_buffers(c, static_cast<std::uint32_t>(want))) return st;
-        if (int st = emit(c, s)) return st;
+    // in the static mode the flag stays up until the host has seen it; otherwise every binning clears it
+    if (int st = bin_lists(c, s, c->depth_mode != XAD_SPLAT_DEPTH_STATIC)) return st;
+    if (check_depth) {
+        XAD_HIP_TRY(hipEventSynchronize(c->report_ready));
+        if (c->report->status[kStatusDepthChanged] != 0) {
+            if (int st = order_by_depth(c, depth, s)) return st;
+            if (int st = project()) return st;  // the rectangles in the new order
+            if (int st = bin_lists(c, s, true)) return st;
+        }
+    }
+    if (!c->capacity_seen) {
+        // The tile-level pair count is exact even when it exceeds the capacity, unless the supertile lists
+        // were cut short as well (then it is a lower bound and the next attempt's count is exact).
+        for (int attempt = 0;; ++attempt) {
+            if (int st = fetch_report(c, s)) return st;
+            if (c->report->status[kStatusOverflow] == 0) break;
+            const std::uint32_t seen = c->pairs > c->report->status[kStatusSuperPairs] ? c->pairs : c->report->status[kStatusSuperPairs];
+            XAD_REQUIRE(attempt < 3 && seen < 0xfffffff0u, "splat: the pair lists overflow at %u pairs", seen);
+            if (int st = size_pair_buffers(c, grown(seen > c->plan.capacity ? seen : c->plan.capacity + 1))) return st;
+            if (int st = bin_lists(c, s, false)) return st;
+        }
+        c->capacity_seen = true;
+        // from now on level A is given only the room this scene needs, with a margin: fewer wavefronts at level B
+        // (an overflow of that margin is reported like any other and resets it)
+        c->plan = make_bin_plan(c->G, c->tiles_x, c->tiles_y, c->plan.capacity, grown(c->report->status[kStatusSuperPairs]));
+        if (int st = clear_status(c, s, kStatusOverflowSticky, 1)) return st;
     }
     mark(c, 2, s);
-    if (int st = sort_pairs(s, c->sort_temp, c->sort_bytes, c->wide_keys, c->keys, c->keys_sorted, c->ids, c->ids_sorted,
-                            c->pairs, c->key_bits))
-        return st;
-    mark(c, 3, s);
-    if (int st = launch_ranges(s, c->pairs, c->wide_keys, c->keys_sorted, c->range_begin, c->range_end)) return st;
-    mark(c, 4, s);
     return XAD_OK;
 }
 
@@ -157,6 +245,29 @@ void collect_times(xad_splat_context* c, int stages) {
     (void)hipEventSynchronize(c->marks[stages]);
     for (int i = 0; i < stages; ++i) (void)hipEventElapsedTime(&c->stage_ms[i], c->marks[i], c->marks[i + 1]);
     for (int i = stages; i < xad_splat_context::kStages; ++i) c->stage_ms[i] = 0.f;
+}
+
+// After a wait: what earlier calls that did not wait have left behind.
+int settle_report(xad_splat_context* c, hipStream_t s, const char* who) {
+    int st = XAD_OK;
+    if (c->depth_mode == XAD_SPLAT_DEPTH_STATIC && c->report->status[kStatusDepthChanged] != 0) {
+        c->order_valid = false;
+        (void)clear_status(c, s, kStatusDepthChanged, 1);
+        st = xad::fail(XAD_ERR_INVALID_ARGUMENT,
+                       "%s: a depth changed although the context is in XAD_SPLAT_DEPTH_STATIC mode; the lists of the calls since "
+                       "then were ordered by the old depths (the order will be recomputed by the next call)",
+                       who);
+    }
+    if (c->report->status[kStatusOverflowSticky] != 0) {
+        const std::uint32_t seen = c->report->status[kStatusOverflowSticky];
+        (void)clear_status(c, s, kStatusOverflowSticky, 1);
+        if (int grow = size_pair_buffers(c, grown(seen > c->plan.capacity ? seen : c->plan.capacity * 2))) return grow;
+        st = xad::fail(XAD_ERR_INCOMPLETE,
+                       "%s: a call that did not wait for the device produced more pairs (%u) than the lists held; its image and "
+                       "gradients were incomplete.  The lists have been enlarged",
+                       who, seen);
+    }
+    return st;
 }
 
 }  // namespace
@@ -182,56 +293,26 @@ extern "C" int xad_splat_create(int width, int height, int num_gaussians, std::s
     c->tiles_x = tiles_x;
     c->tiles_y = tiles_y;
     c->tiles = tiles_x * tiles_y;
-    int tile_bits = 1;
-    while ((1 << tile_bits) < c->tiles) ++tile_bits;
-    c->key_bits = tile_bits;
-    c->wide_keys = c->tiles > 65536;
-    const std::size_t pixels = static_cast<std::size_t>(width) * height;
-    const std::size_t G = static_cast<std::size_t>(num_gaussians);
+    c->depth_sort_bytes = depth_sort_temp_bytes(num_gaussians);
     int st = XAD_OK;
-    auto alloc = [&](auto** p, std::size_t bytes) {
-        if (st == XAD_OK && hipMalloc(reinterpret_cast<void**>(p), bytes) != hipSuccess)
-            st = xad::fail(XAD_ERR_HIP, "%s: hipMalloc of %zu bytes failed", who, bytes);
-    };
-    alloc(&c->records, sizeof(Record) * G);
-    alloc(&c->rects, sizeof(TileRect) * G);
-    alloc(&c->depth_keys, sizeof(std::uint32_t) * G);
-    alloc(&c->depth_keys_sorted, sizeof(std::uint32_t) * G);
-    alloc(&c->identity, sizeof(std::uint32_t) * G);
-    alloc(&c->by_depth, sizeof(std::uint32_t) * G);
-    alloc(&c->counts_by_depth, sizeof(std::uint32_t) * (G + 1));
-    alloc(&c->counts, sizeof(std::uint32_t) * (G + 1));
-    alloc(&c->offsets, sizeof(std::uint32_t) * (G + 2));
-    alloc(&c->ordered_depth, sizeof(float) * G);
-    alloc(&c->range_begin, sizeof(std::uint32_t) * c->tiles * 2);
-    alloc(&c->final_T, sizeof(float) * pixels);
-    alloc(&c->n_contrib, sizeof(std::uint32_t) * pixels);
-    alloc(&c->record_grads, sizeof(float) * G * kRecordGradStride);
-    alloc(&c->loss, sizeof(double));
+    std::size_t bytes = 0;
+    carve_fixed(c, nullptr, &bytes);
+    if (hipMalloc(&c->fixed, bytes) != hipSuccess) st = xad::fail(XAD_ERR_HIP, "%s: hipMalloc of %zu bytes failed", who, bytes);
     if (st == XAD_OK) {
-        c->range_end = c->range_begin + c->tiles;
-        c->scan_bytes = scan_temp_bytes(num_gaussians);
-        alloc(&c->scan_temp, c->scan_bytes ? c->scan_bytes : 16);
-        c->depth_sort_bytes = depth_sort_temp_bytes(num_gaussians);
-        alloc(&c->depth_sort_temp, c->depth_sort_bytes ? c->depth_sort_bytes : 16);
+        carve_fixed(c, static_cast<char*>(c->fixed), &bytes);
+        // status words, the scan's ticket counter and the tile ranges start from zero
+        if (hipMemset(c->fixed, 0, bytes) != hipSuccess) st = xad::fail(XAD_ERR_HIP, "%s: hipMemset failed", who);
     }
-    if (st == XAD_OK && hipHostMalloc(reinterpret_cast<void**>(&c->host_pairs), 2 * sizeof(std::uint32_t)) != hipSuccess)
+    if (st == XAD_OK && hipHostMalloc(reinterpret_cast<void**>(&c->report), sizeof(HostReport)) != hipSuccess)
         st = xad::fail(XAD_ERR_HIP, "%s: pinned allocation failed", who);
-    if (st == XAD_OK && hipHostMalloc(reinterpret_cast<void**>(&c->host_loss), sizeof(double)) != hipSuccess)
-        st = xad::fail(XAD_ERR_HIP, "%s: pinned allocation failed", who);
-    if (st == XAD_OK && hipMemset(c->counts, 0, sizeof(std::uint32_t) * (G + 1)) != hipSuccess)
-        st = xad::fail(XAD_ERR_HIP, "%s: hipMemset failed", who);
-    if (st == XAD_OK && hipMemset(c->counts_by_depth, 0, sizeof(std::uint32_t) * (G + 1)) != hipSuccess)
-        st = xad::fail(XAD_ERR_HIP, "%s: hipMemset failed", who);
-    if (st == XAD_OK && hipMemset(c->offsets, 0, sizeof(std::uint32_t) * (G + 2)) != hipSuccess)  // includes the flag
-        st = xad::fail(XAD_ERR_HIP, "%s: hipMemset failed", who);
     if (st == XAD_OK) {
-        const std::size_t hint = pair_capacity_hint ? pair_capacity_hint : G * 8 + 1024;
-        st = allocate_pair_buffers(c, static_cast<std::uint32_t>(hint < 0xfffffff0ull ? hint : 0xfffffff0ull));
+        *c->report = HostReport{};
+        const std::size_t hint = pair_capacity_hint ? pair_capacity_hint : static_cast<std::size_t>(num_gaussians) * 8 + 1024;
+        st = size_pair_buffers(c, static_cast<std::uint32_t>(hint < 0xfffffff0ull ? hint : 0xfffffff0ull));
     }
     for (auto& e : c->marks)
         if (st == XAD_OK && hipEventCreate(&e) != hipSuccess) st = xad::fail(XAD_ERR_HIP, "%s: hipEventCreate failed", who);
-    if (st == XAD_OK && hipEventCreateWithFlags(&c->count_ready, hipEventDisableTiming) != hipSuccess)
+    if (st == XAD_OK && hipEventCreateWithFlags(&c->report_ready, hipEventDisableTiming) != hipSuccess)
         st = xad::fail(XAD_ERR_HIP, "%s: hipEventCreate failed", who);
     if (st != XAD_OK) {
         xad_splat_destroy(c);
@@ -243,29 +324,12 @@ extern "C" int xad_splat_create(int width, int height, int num_gaussians, std::s
 
 extern "C" void xad_splat_destroy(xad_splat_context* c) {
     if (!c) return;
-    free_pair_buffers(c);
-    (void)hipFree(c->records);
-    (void)hipFree(c->rects);
-    (void)hipFree(c->depth_keys);
-    (void)hipFree(c->depth_keys_sorted);
-    (void)hipFree(c->identity);
-    (void)hipFree(c->by_depth);
-    (void)hipFree(c->counts_by_depth);
-    (void)hipFree(c->ordered_depth);
-    (void)hipFree(c->depth_sort_temp);
-    (void)hipFree(c->counts);
-    (void)hipFree(c->offsets);
-    (void)hipFree(c->range_begin);
-    (void)hipFree(c->final_T);
-    (void)hipFree(c->n_contrib);
-    (void)hipFree(c->record_grads);
-    (void)hipFree(c->loss);
-    (void)hipFree(c->scan_temp);
-    if (c->host_pairs) (void)hipHostFree(c->host_pairs);
-    if (c->host_loss) (void)hipHostFree(c->host_loss);
+    if (c->paired) (void)hipFree(c->paired);
+    if (c->fixed) (void)hipFree(c->fixed);
+    if (c->report) (void)hipHostFree(c->report);
     for (auto& e : c->marks)
         if (e) (void)hipEventDestroy(e);
-    if (c->count_ready) (void)hipEventDestroy(c->count_ready);
+    if (c->report_ready) (void)hipEventDestroy(c->report_ready);
     delete c;
 }
 
@@ -275,17 +339,26 @@ extern "C" int xad_splat_set_profiling(xad_splat_context* c, int enabled) {
     return XAD_OK;
 }
 
+extern "C" int xad_splat_set_depth_mode(xad_splat_context* c, int mode) {
+    XAD_REQUIRE(c, "xad_splat_set_depth_mode: context is null");
+    XAD_REQUIRE(mode == XAD_SPLAT_DEPTH_CHECKED || mode == XAD_SPLAT_DEPTH_STATIC || mode == XAD_SPLAT_DEPTH_EVERY_STEP,
+                "xad_splat_set_depth_mode: unknown mode %d", mode);
+    c->depth_mode = mode;
+    c->order_valid = false;  // the next call orders by the depths it is given
+    return XAD_OK;
+}
+
 extern "C" int xad_splat_forward(xad_splat_context* c, const float* params, const float* depth, float* image,
                                  void* stream) {
     const char* who = "xad_splat_forward";
     XAD_REQUIRE(c && params && depth && image, "%s: null argument", who);
     hipStream_t s = xad::as_stream(stream);
     if (int st = bin(c, params, depth, s)) return st;
-    if (int st = launch_render_forward(s, c->width, c->height, c->range_begin, c->range_end, c->ids_sorted, c->records,
-                                       image, c->final_T, c->n_contrib))
+    if (int st = launch_render_forward(s, c->width, c->height, c->range_begin, c->range_end, c->list, c->records, image,
+                                       c->final_T, c->n_contrib))
         return st;
-    mark(c, 5, s);
-    collect_times(c, 5);
+    mark(c, 3, s);
+    collect_times(c, 3);
     return XAD_OK;
 }
 
@@ -294,33 +367,50 @@ extern "C" int xad_splat_step(xad_splat_context* c, const float* params, const f
     const char* who = "xad_splat_step";
     XAD_REQUIRE(c && params && depth && target && image && grads, "%s: null argument", who);
     hipStream_t s = xad::as_stream(stream);
-    if (int st = bin(c, params, depth, s)) return st;
-    if (int st = launch_render_forward(s, c->width, c->height, c->range_begin, c->range_end, c->ids_sorted, c->records,
-                                       image, c->final_T, c->n_contrib))
-        return st;
-    mark(c, 5, s);
-    if (int st = launch_render_backward(s, c->width, c->height, c->range_begin, c->range_end, c->ids_sorted, c->records,
-                                        image, target, c->final_T, c->n_contrib, c->record_grads, c->loss))
-        return st;
-    mark(c, 6, s);
-    if (int st = launch_gaussian_backward(s, c->G, params, c->record_grads, grads)) return st;
-    mark(c, 7, s);
-    if (loss_out) {
-        XAD_HIP_TRY(hipMemcpyAsync(c->host_loss, c->loss, sizeof(double), hipMemcpyDeviceToHost, s));
-        XAD_HIP_TRY(hipStreamSynchronize(s));
-        *loss_out = *c->host_loss;
+    for (int attempt = 0;; ++attempt) {
+        if (int st = bin(c, params, depth, s)) return st;
+        if (int st = launch_render_forward(s, c->width, c->height, c->range_begin, c->range_end, c->list, c->records, image,
+                                           c->final_T, c->n_contrib))
+            return st;
+        mark(c, 3, s);
+        if (int st = launch_render_backward(s, c->width, c->height, c->range_begin, c->range_end, c->list, c->records, image,
+                                            target, c->final_T, c->n_contrib, c->record_grads, c->loss))
+            return st;
+        mark(c, 4, s);
+        if (int st = launch_gaussian_backward(s, c->G, params, c->record_grads, grads)) return st;
+        mark(c, 5, s);
+        if (!loss_out) break;
+        // the loss is read back, and with it what the device has to report
+        if (int st = fetch_report(c, s)) return st;
+        if (c->report->status[kStatusOverflow] != 0 && attempt == 0) {
+            // this very step did not fit (the scene grew): enlarge the lists and do it again
+            if (int st = size_pair_buffers(c, grown(c->pairs > c->plan.capacity ? c->pairs : c->plan.capacity * 2))) return st;
+            if (int st = clear_status(c, s, kStatusOverflowSticky, 1)) return st;
+            c->report->status[kStatusOverflowSticky] = 0;
+            continue;
+        }
+        *loss_out = c->report->loss;
+        if (int st = settle_report(c, s, who)) {
+            collect_times(c, 5);
+            return st;
+        }
+        break;
     }
-    collect_times(c, 7);
+    collect_times(c, 5);
     return XAD_OK;
 }
 
-extern "C" int xad_splat_get_stats(const xad_splat_context* c, std::uint64_t* pairs, std::uint32_t* longest_list,
-                                   float* stage_ms) {
+extern "C" int xad_splat_get_stats(xad_splat_context* c, std::uint64_t* pairs, std::uint32_t* longest_list, float* stage_ms) {
     const char* who = "xad_splat_get_stats";
     XAD_REQUIRE(c, "%s: context is null", who);
+    if (pairs || longest_list) {
+        // waits for everything queued on the device, then reads the status words of the last step
+        XAD_HIP_TRY(hipDeviceSynchronize());
+        XAD_HIP_TRY(hipMemcpy(c->report->status, c->status, sizeof(std::uint32_t) * kStatusWords, hipMemcpyDeviceToHost));
+        c->pairs = c->report->status[kStatusPairs];
+    }
     if (pairs) *pairs = c->pairs;
     if (longest_list) {
-        // computed on demand from the tile ranges of the last step
         std::uint32_t* host = new (std::nothrow) std::uint32_t[static_cast<std::size_t>(c->tiles) * 2];
         XAD_REQUIRE(host, "%s: out of host memory", who);
         hipError_t e = hipMemcpy(host, c->range_begin, sizeof(std::uint32_t) * c->tiles * 2, hipMemcpyDeviceToHost);
@@ -336,5 +426,22 @@ extern "C" int xad_splat_get_stats(const xad_splat_context* c, std::uint64_t* pa
     }
     if (stage_ms)
         for (int i = 0; i < xad_splat_context::kStages; ++i) stage_ms[i] = c->stage_ms[i];
+    return XAD_OK;
+}
+
+extern "C" int xad_splat_get_lists(xad_splat_context* c, std::uint32_t* range_begin, std::uint32_t* range_end,
+                                   std::uint32_t* gaussians, std::size_t capacity) {
+    const char* who = "xad_splat_get_lists";
+    XAD_REQUIRE(c && range_begin && range_end, "%s: null argument", who);
+    XAD_HIP_TRY(hipDeviceSynchronize());
+    XAD_HIP_TRY(hipMemcpy(c->report->status, c->status, sizeof(std::uint32_t) * kStatusWords, hipMemcpyDeviceToHost));
+    c->pairs = c->report->status[kStatusPairs];
+    XAD_REQUIRE(c->report->status[kStatusOverflow] == 0, "%s: the last step's lists overflowed", who);
+    XAD_HIP_TRY(hipMemcpy(range_begin, c->range_begin, sizeof(std::uint32_t) * c->tiles, hipMemcpyDeviceToHost));
+    XAD_HIP_TRY(hipMemcpy(range_end, c->range_end, sizeof(std::uint32_t) * c->tiles, hipMemcpyDeviceToHost));
+    if (gaussians) {
+        XAD_REQUIRE(capacity >= c->pairs, "%s: room for %zu entries, the lists hold %u", who, capacity, c->pairs);
+        if (c->pairs) XAD_HIP_TRY(hipMemcpy(gaussians, c->list, sizeof(std::uint32_t) * c->pairs, hipMemcpyDeviceToHost));
+    }
     return XAD_OK;
 }

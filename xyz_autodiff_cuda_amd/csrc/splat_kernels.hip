@@ -1,6 +1,6 @@
-// Kernels of the tile-binned splatting step: per-Gaussian projection, pair
-// emission, tile ranges, per-tile compositing forward and reverse-order
-// backward, per-Gaussian parameter backward.
+// Kernels of the tile-binned splatting step: per-Gaussian projection, per-tile
+// compositing forward and reverse-order backward, per-Gaussian parameter
+// backward.  (The tile lists come from splat_binning.hip.)
 //
 // Every kernel is HBM-, LDS- or VALU-bound streaming work on small records;
 // nothing here is a dense contraction.
@@ -27,13 +27,14 @@ using namespace xyz_autodiff;
 //   es = exp(log-scale); cov = scale_rotation_to_covariance_3param(es, theta);
 //   inv = sym_matrix2_inv(cov); alpha0 = sigmoid(opacity)
 // from the library's nodes, runs it forward, and derives the 3-sigma tile
-// rectangle and the number of tiles.
+// rectangle.
 __global__ void __launch_bounds__(256) project_kernel(int G, const float* __restrict__ params,
                                                       const float* __restrict__ depth,
                                                       const float* __restrict__ ordered_depth,
-                                                      std::uint32_t* __restrict__ depth_changed, int width, int height,
+                                                      const std::uint32_t* __restrict__ rank,
+                                                      std::uint32_t* __restrict__ status, int width, int height,
                                                       Record* __restrict__ records, TileRect* __restrict__ rects,
-                                                      std::uint32_t* __restrict__ counts,
+                                                      TileRect* __restrict__ rects_by_depth,
                                                       float* __restrict__ record_grads, double* __restrict__ loss) {
     const int g = blockIdx.x * 256 + threadIdx.x;
     if (g >= G) return;
@@ -46,7 +47,7 @@ __global__ void __launch_bounds__(256) project_kernel(int G, const float* __rest
     }
     // the depth order of the previous call stays valid while every depth keeps its bits
     if (__builtin_bit_cast(std::uint32_t, depth[g]) != __builtin_bit_cast(std::uint32_t, ordered_depth[g]))
-        atomicOr(depth_changed, 1u);
+        atomicOr(status + kStatusDepthChanged, 1u);
     const std::size_t n = static_cast<std::size_t>(G);
     const float cx = params[0 * n + g], cy = params[1 * n + g];
     Variable<2, float> log_scale;
@@ -78,7 +79,6 @@ __global__ void __launch_bounds__(256) project_kernel(int G, const float* __rest
     const int tiles_x = (width + kTile - 1) / kTile, tiles_y = (height + kTile - 1) / kTile;
     const float rx = 3.f * ::sqrtf(cov[0]), ry = 3.f * ::sqrtf(cov[2]);
     TileRect rc{1, 1, 0, 0};
-    std::uint32_t count = 0;
     const bool finite = ::isfinite(cx) && ::isfinite(cy) && ::isfinite(rx) && ::isfinite(ry) && ::isfinite(rec.a) &&
                         ::isfinite(rec.b) && ::isfinite(rec.c) && ::isfinite(rec.alpha0);
     if (finite) {
@@ -89,11 +89,10 @@ __global__ void __launch_bounds__(256) project_kernel(int G, const float* __rest
             rc.y0 = static_cast<std::int16_t>(lo_y < 0.f ? 0 : static_cast<int>(lo_y));
             rc.x1 = static_cast<std::int16_t>(hi_x > static_cast<float>(tiles_x - 1) ? tiles_x - 1 : static_cast<int>(hi_x));
             rc.y1 = static_cast<std::int16_t>(hi_y > static_cast<float>(tiles_y - 1) ? tiles_y - 1 : static_cast<int>(hi_y));
-            count = static_cast<std::uint32_t>(rc.x1 - rc.x0 + 1) * static_cast<std::uint32_t>(rc.y1 - rc.y0 + 1);
         }
     }
     rects[g] = rc;
-    counts[g] = count;
+    rects_by_depth[rank[g]] = rc;  // the binning walks the Gaussians in depth order
 }
 
 // Order-preserving map from float to unsigned (any sign).
@@ -102,11 +101,16 @@ __device__ __forceinline__ std::uint32_t ordered_bits(float f) {
     return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
 }
 
+__global__ void __launch_bounds__(256) depth_rank_kernel(int G, const std::uint32_t* __restrict__ by_depth,
+                                                         std::uint32_t* __restrict__ rank) {
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i < G) rank[by_depth[i]] = static_cast<std::uint32_t>(i);
+}
+
 // Depth order.  depth_key_kernel writes the order-preserving bits of every depth
 // and the identity permutation; a stable sort of those pairs gives by_depth, the
-// Gaussians in (depth, index) order.  Pairs are then emitted in that order, so a
-// stable sort on the tile index alone leaves every tile's list in depth order:
-// the pair sort handles 16-bit (or 32-bit) keys instead of tile | depth.
+// Gaussians in (depth, index) order.  The binning walks the Gaussians in that
+// order, which leaves every tile's list in depth order without sorting pairs.
 __global__ void __launch_bounds__(256) depth_key_kernel(int G, const float* __restrict__ depth,
                                                         std::uint32_t* __restrict__ keys,
                                                         std::uint32_t* __restrict__ identity) {
@@ -114,86 +118,6 @@ __global__ void __launch_bounds__(256) depth_key_kernel(int G, const float* __re
     if (g >= G) return;
     keys[g] = ordered_bits(depth[g]);
     identity[g] = static_cast<std::uint32_t>(g);
-}
-
-// counts in depth order, the input of the scan that places the pairs
-__global__ void __launch_bounds__(256) permute_counts_kernel(int G, const std::uint32_t* __restrict__ by_depth,
-                                                             const std::uint32_t* __restrict__ counts,
-                                                             std::uint32_t* __restrict__ counts_by_depth) {
-    const int i = blockIdx.x * 256 + threadIdx.x;
-    if (i >= G) return;
-    counts_by_depth[i] = counts[by_depth[i]];
-}
-
-// Pair emission: the i-th Gaussian in depth order writes one (tile, index) pair
-// per tile of its rectangle into the segment [offsets[i], offsets[i+1]).  A lane
-// writes a small rectangle by itself; a large one (up to hundreds of tiles) is
-// written by its whole wavefront, lane t taking every 64th tile, so the stores
-// are coalesced and no lane is left walking a long rectangle alone.
-constexpr std::uint32_t kEmitAlone = 8;
-
-template <typename Key>
-__global__ void __launch_bounds__(256) emit_kernel(int G, const std::uint32_t* __restrict__ by_depth,
-                                                   const TileRect* __restrict__ rects,
-                                                   const std::uint32_t* __restrict__ offsets, int tiles_x,
-                                                   Key* __restrict__ keys, std::uint32_t* __restrict__ values,
-                                                   std::uint32_t capacity, std::uint32_t* __restrict__ tile_ranges,
-                                                   int range_words, std::uint32_t* __restrict__ depth_changed) {
-    const int i = blockIdx.x * 256 + threadIdx.x;
-    const int lane = threadIdx.x & 63;
-    // housekeeping for what runs later in the step: empty tile ranges (tiles without pairs keep
-    // them), and the depth-changed flag, which the host has read by now, back to zero
-    for (int t = i; t < range_words; t += static_cast<int>(gridDim.x) * 256) tile_ranges[t] = 0;
-    if (i == 0) *depth_changed = 0;
-    std::uint32_t g = 0, at = 0, count = 0;
-    int x0 = 0, y0 = 0, columns = 1;
-    if (i < G) {
-        g = by_depth[i];
-        const TileRect rc = rects[g];
-        if (rc.x0 <= rc.x1) {
-            x0 = rc.x0;
-            y0 = rc.y0;
-            columns = rc.x1 - rc.x0 + 1;
-            count = static_cast<std::uint32_t>(columns) * static_cast<std::uint32_t>(rc.y1 - rc.y0 + 1);
-            at = offsets[i];
-        }
-    }
-    if (count <= kEmitAlone) {
-        for (std::uint32_t t = 0; t < count; ++t) {
-            const int ty = y0 + static_cast<int>(t) / columns, tx = x0 + static_cast<int>(t) % columns;
-            if (at + t < capacity) {
-                keys[at + t] = static_cast<Key>(ty * tiles_x + tx);
-                values[at + t] = g;
-            }
-        }
-    }
-    // every lane of the wavefront reaches this loop: the large rectangles are taken one by one
-    for (std::uint64_t large = accumulate::wave::ballot(count > kEmitAlone); large != 0; large &= large - 1) {
-        const int owner = __builtin_ctzll(large);
-        const std::uint32_t n = __builtin_amdgcn_readlane(count, owner), first = __builtin_amdgcn_readlane(at, owner);
-        const std::uint32_t id = __builtin_amdgcn_readlane(g, owner);
-        const int c = __builtin_amdgcn_readlane(columns, owner);
-        const int bx = __builtin_amdgcn_readlane(x0, owner), by = __builtin_amdgcn_readlane(y0, owner);
-        for (std::uint32_t t = lane; t < n; t += 64) {
-            const int ty = by + static_cast<int>(t) / c, tx = bx + static_cast<int>(t) % c;
-            if (first + t < capacity) {
-                keys[first + t] = static_cast<Key>(ty * tiles_x + tx);
-                values[first + t] = id;
-            }
-        }
-    }
-}
-
-// Tile ranges from the sorted keys: ranges[t] = [first, last) positions of tile t.
-template <typename Key>
-__global__ void __launch_bounds__(256) ranges_kernel(std::uint32_t K, const Key* __restrict__ keys,
-                                                     std::uint32_t* __restrict__ range_begin,
-                                                     std::uint32_t* __restrict__ range_end) {
-    const std::uint32_t i = blockIdx.x * 256u + threadIdx.x;
-    if (i >= K) return;
-    const std::uint32_t t = keys[i];
-    if (i == 0 || keys[i - 1] != keys[i]) range_begin[t] = i;
-    if (i + 1 == K || keys[i + 1] != keys[i]) range_end[t] = i + 1;
 }
 
 // Blocks are handed to the eight XCDs round-robin; giving each XCD a contiguous
@@ -657,52 +581,22 @@ __global__ void __launch_bounds__(256) gaussian_backward_kernel(int G, const flo
 // launchers (declared in splat_launch.cuh)
 
 int launch_project(hipStream_t s, int G, const float* params, const float* depth, const float* ordered_depth,
-                   std::uint32_t* depth_changed, int width, int height, Record* records, TileRect* rects,
-                   std::uint32_t* counts, float* record_grads, double* loss) {
-    hipLaunchKernelGGL(project_kernel, dim3(xad::blocks_for(G, 256)), dim3(256), 0, s, G, params, depth, ordered_depth,
-                       depth_changed, width, height, records, rects, counts, record_grads, loss);
+                   const std::uint32_t* rank, std::uint32_t* status, int width, int height, Record* records, TileRect* rects,
+                   TileRect* rects_by_depth, float* record_grads, double* loss) {
+    hipLaunchKernelGGL(project_kernel, dim3(xad::blocks_for(G, 256)), dim3(256), 0, s, G, params, depth, ordered_depth, rank,
+                       status, width, height, records, rects, rects_by_depth, record_grads, loss);
+    XAD_HIP_TRY(hipGetLastError());
+    return XAD_OK;
+}
+
+int launch_depth_rank(hipStream_t s, int G, const std::uint32_t* by_depth, std::uint32_t* rank) {
+    hipLaunchKernelGGL(depth_rank_kernel, dim3(xad::blocks_for(G, 256)), dim3(256), 0, s, G, by_depth, rank);
     XAD_HIP_TRY(hipGetLastError());
     return XAD_OK;
 }
 
 int launch_depth_keys(hipStream_t s, int G, const float* depth, std::uint32_t* keys, std::uint32_t* identity) {
     hipLaunchKernelGGL(depth_key_kernel, dim3(xad::blocks_for(G, 256)), dim3(256), 0, s, G, depth, keys, identity);
-    XAD_HIP_TRY(hipGetLastError());
-    return XAD_OK;
-}
-
-int launch_permute_counts(hipStream_t s, int G, const std::uint32_t* by_depth, const std::uint32_t* counts,
-                          std::uint32_t* counts_by_depth) {
-    hipLaunchKernelGGL(permute_counts_kernel, dim3(xad::blocks_for(G, 256)), dim3(256), 0, s, G, by_depth, counts,
-                       counts_by_depth);
-    XAD_HIP_TRY(hipGetLastError());
-    return XAD_OK;
-}
-
-int launch_emit(hipStream_t s, int G, const std::uint32_t* by_depth, const TileRect* rects, const std::uint32_t* offsets,
-                int tiles_x, bool wide_keys, void* keys, std::uint32_t* values, std::uint32_t capacity,
-                std::uint32_t* tile_ranges, int range_words, std::uint32_t* depth_changed) {
-    if (wide_keys)
-        hipLaunchKernelGGL(emit_kernel<std::uint32_t>, dim3(xad::blocks_for(G, 256)), dim3(256), 0, s, G, by_depth, rects,
-                           offsets, tiles_x, static_cast<std::uint32_t*>(keys), values, capacity, tile_ranges, range_words,
-                           depth_changed);
-    else
-        hipLaunchKernelGGL(emit_kernel<std::uint16_t>, dim3(xad::blocks_for(G, 256)), dim3(256), 0, s, G, by_depth, rects,
-                           offsets, tiles_x, static_cast<std::uint16_t*>(keys), values, capacity, tile_ranges, range_words,
-                           depth_changed);
-    XAD_HIP_TRY(hipGetLastError());
-    return XAD_OK;
-}
-
-int launch_ranges(hipStream_t s, std::uint32_t K, bool wide_keys, const void* keys, std::uint32_t* range_begin,
-                  std::uint32_t* range_end) {
-    if (K == 0) return XAD_OK;
-    if (wide_keys)
-        hipLaunchKernelGGL(ranges_kernel<std::uint32_t>, dim3(xad::blocks_for(K, 256)), dim3(256), 0, s, K,
-                           static_cast<const std::uint32_t*>(keys), range_begin, range_end);
-    else
-        hipLaunchKernelGGL(ranges_kernel<std::uint16_t>, dim3(xad::blocks_for(K, 256)), dim3(256), 0, s, K,
-                           static_cast<const std::uint16_t*>(keys), range_begin, range_end);
     XAD_HIP_TRY(hipGetLastError());
     return XAD_OK;
 }

@@ -1,7 +1,6 @@
 #pragma once
-// Host-callable launchers of the splatting kernels and of the scan/sort stage,
-// so that the translation unit that instantiates the device-wide primitives is
-// compiled separately from the hand-written kernels.
+// Host-callable launchers of the splatting kernels, of the binning stage and of the depth sort, each
+// in a translation unit of its own.
 #include <hip/hip_runtime.h>
 
 #include <cstddef>
@@ -11,24 +10,61 @@
 
 namespace xad_splat {
 
-// Also sets *depth_changed to 1 if any depth differs (bitwise) from ordered_depth, and zeroes
+// Words of the step's status block on the device (read by the host whenever it next waits for the stream).
+enum : int {
+    kStatusPairs = 0,         // (tile, Gaussian) pairs of the last binning
+    kStatusOverflow = 1,      // 1 if the pairs did not fit the lists: the lists of that step are incomplete
+    kStatusSuperPairs = 2,    // (supertile, Gaussian) pairs
+    kStatusDepthChanged = 3,  // 1 if a depth differed from the depths the kept order was computed from
+    kStatusOverflowSticky = 4,  // largest pair count of any step that overflowed since the host last cleared this word
+    kStatusWords = 5,
+};
+
+// Also sets status[kStatusDepthChanged] if any depth differs (bitwise) from ordered_depth, and zeroes
 // record_grads (G rows of kRecordGradStride floats) and *loss for the compositing backward.
+// rank[g] = position of Gaussian g in the depth order: the rectangle is also written to rects_by_depth[rank[g]].
 int launch_project(hipStream_t s, int G, const float* params, const float* depth, const float* ordered_depth,
-                   std::uint32_t* depth_changed, int width, int height, Record* records, TileRect* rects,
-                   std::uint32_t* counts, float* record_grads, double* loss);
+                   const std::uint32_t* rank, std::uint32_t* status, int width, int height, Record* records, TileRect* rects,
+                   TileRect* rects_by_depth, float* record_grads, double* loss);
 // Depth order: keys[g] = order-preserving bits of depth[g], identity[g] = g; the stable sort of
-// those pairs gives by_depth.  counts_by_depth[i] = counts[by_depth[i]].
+// those pairs gives by_depth; rank is its inverse (rank[by_depth[i]] = i).
 int launch_depth_keys(hipStream_t s, int G, const float* depth, std::uint32_t* keys, std::uint32_t* identity);
-int launch_permute_counts(hipStream_t s, int G, const std::uint32_t* by_depth, const std::uint32_t* counts,
-                          std::uint32_t* counts_by_depth);
-// Pairs are emitted in depth order with the tile index as key: 16 bits wide, or 32 (wide_keys)
-// when there are more than 65 536 tiles.
-// Also zeroes the range_words words of tile_ranges and resets *depth_changed.
-int launch_emit(hipStream_t s, int G, const std::uint32_t* by_depth, const TileRect* rects, const std::uint32_t* offsets,
-                int tiles_x, bool wide_keys, void* keys, std::uint32_t* values, std::uint32_t capacity,
-                std::uint32_t* tile_ranges, int range_words, std::uint32_t* depth_changed);
-int launch_ranges(hipStream_t s, std::uint32_t K, bool wide_keys, const void* keys, std::uint32_t* range_begin,
-                  std::uint32_t* range_end);
+int launch_depth_rank(hipStream_t s, int G, const std::uint32_t* by_depth, std::uint32_t* rank);
+
+// Binning (splat_binning.hip): tile lists from tile rectangles, Gaussians taken in the order by_depth.
+constexpr std::uint32_t kBinRangeB = 64;  // list entries a wavefront handles at level B: one per lane
+struct BinPlan {
+    int G, tiles_x, tiles_y;
+    int super_x, super_y, supers;  // supertiles of 8 x 8 tiles
+    int groups;                    // groups of 64 supertiles
+    int range_a, ranges_a;         // Gaussians per wavefront at level A, and how many such ranges
+    std::uint32_t capacity;        // (tile, Gaussian) pairs the lists can hold
+    std::uint32_t capacity_a;      // (supertile, Gaussian) pairs level A may produce: at most capacity (the buffer's size)
+    std::uint32_t waves_b;         // wavefronts launched at level B: capacity_a / kBinRangeB + supers
+};
+struct BinScratch {
+    std::uint32_t* matrix_a = nullptr;    // bin_matrix_a_words: counts, then offsets, per (supertile, range)
+    std::uint32_t* matrix_b = nullptr;    // bin_matrix_b_words: the same per (tile, range of its supertile's list)
+    std::uint32_t* list_a = nullptr;      // capacity: the supertiles' lists
+    std::uint32_t* first_wave = nullptr;  // supers + 1
+    std::uint64_t* scan_state = nullptr;  // bin_scan_state_words, zero before the first launch
+    std::uint32_t* tickets = nullptr;     // one word, zero before the first launch
+    std::uint32_t tickets_taken = 0;      // host mirror of *tickets
+    std::uint32_t epoch = 0;              // of the last scan launched
+};
+// The buffers are sized by a plan with capacity_a = capacity; a plan with a smaller capacity_a (once the host
+// has seen how many supertile pairs a scene produces) uses less of them and launches fewer wavefronts.
+BinPlan make_bin_plan(int G, int tiles_x, int tiles_y, std::uint32_t capacity, std::uint32_t capacity_a);
+std::size_t bin_matrix_a_words(const BinPlan& p);
+std::size_t bin_matrix_b_words(const BinPlan& p);
+std::size_t bin_scan_state_words(const BinPlan& p);
+// Fills list (capacity entries), range_begin / range_end (one entry per tile, adjacent arrays) and
+// status[kStatusPairs, kStatusOverflow, kStatusSuperPairs]; clears status[kStatusDepthChanged] when asked to.
+// rects_by_depth[i] = rects[by_depth[i]].
+int launch_binning(hipStream_t s, const BinPlan& p, const std::uint32_t* by_depth, const TileRect* rects_by_depth,
+                   const TileRect* rects, BinScratch& scratch,
+                   std::uint32_t* list, std::uint32_t* range_begin, std::uint32_t* range_end, std::uint32_t* status,
+                   bool clear_depth_flag);
 int launch_render_forward(hipStream_t s, int width, int height, const std::uint32_t* range_begin,
                           const std::uint32_t* range_end, const std::uint32_t* sorted_ids, const Record* records,
                           float* image, float* final_T, std::uint32_t* n_contrib);
@@ -38,18 +74,9 @@ int launch_render_backward(hipStream_t s, int width, int height, const std::uint
                            const std::uint32_t* n_contrib, float* record_grads, double* loss);
 int launch_gaussian_backward(hipStream_t s, int G, const float* params, const float* record_grads, float* grads);
 
-// Device-wide primitives (rocPRIM): exclusive scan of the per-Gaussian tile
-// counts (offsets has G + 1 entries, the last is the number of pairs), the
-// stable radix sort of (depth bits, index) that yields the depth order, and the
-// stable radix sort of the (tile, index) pairs over the `key_bits` bits of a tile index.
-std::size_t scan_temp_bytes(int G);
-int exclusive_scan_counts(hipStream_t s, void* temp, std::size_t temp_bytes, const std::uint32_t* counts,
-                          std::uint32_t* offsets, int G);
+// The stable radix sort of (depth bits, index) that yields the depth order (rocPRIM; runs only when a depth changed).
 std::size_t depth_sort_temp_bytes(int G);
 int sort_by_depth(hipStream_t s, void* temp, std::size_t temp_bytes, const std::uint32_t* keys_in,
                   std::uint32_t* keys_out, const std::uint32_t* values_in, std::uint32_t* values_out, int G);
-std::size_t sort_temp_bytes(std::uint32_t capacity, bool wide_keys);
-int sort_pairs(hipStream_t s, void* temp, std::size_t temp_bytes, bool wide_keys, const void* keys_in, void* keys_out,
-               const std::uint32_t* values_in, std::uint32_t* values_out, std::uint32_t K, int key_bits);
 
 }  // namespace xad_splat

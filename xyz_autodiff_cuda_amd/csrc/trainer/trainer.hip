@@ -87,6 +87,8 @@ int create(const xad_training_config* config, int width, int height, const float
     XAD_HIP_TRY(hipGetDevice(&t->device));
     XAD_HIP_TRY(hipStreamCreate(&t->stream));
     if (int st = xad_splat_create(width, height, t->gaussians, 0, &t->splat)) return st;
+    // depth is drawn once and never trained: promise that, so that an iteration never waits for the device
+    if (int st = xad_splat_set_depth_mode(t->splat, XAD_SPLAT_DEPTH_STATIC)) return st;
     XAD_HIP_TRY(hipMalloc(&t->state, 37 * t->g() * sizeof(float)));
     XAD_HIP_TRY(hipMalloc(&t->target, 3 * t->pixels() * sizeof(float)));
     XAD_HIP_TRY(hipMalloc(&t->image, 3 * t->pixels() * sizeof(float)));

@@ -10,7 +10,8 @@ import math
 from . import _lib, rng
 
 PARAM_ROWS = ("cx", "cy", "log_sx", "log_sy", "theta", "r", "g", "b", "opacity")
-STAGES = ("project", "scan_emit", "sort", "tile_ranges", "render_forward", "render_backward", "parameter_backward")
+STAGES = ("project", "binning", "render_forward", "render_backward", "parameter_backward")
+DEPTH_MODES = {"checked": 0, "static": 1, "every_step": 2}
 
 
 def _check_tensor(t, shape, name, dtype=None):
@@ -24,7 +25,10 @@ def _check_tensor(t, shape, name, dtype=None):
 class SplatContext:
     """Owns the device workspace of the step for one image size and Gaussian count."""
 
-    def __init__(self, width, height, num_gaussians, pair_capacity_hint=0, device=None):
+    def __init__(self, width, height, num_gaussians, pair_capacity_hint=0, device=None, depth_mode="checked"):
+        """depth_mode: "checked" (every call looks whether a depth changed since the Gaussians were last ordered:
+        one wait per call), "static" (a promise that depth does not change: calls that do not ask for the loss
+        only queue work) or "every_step" (the order is recomputed by every call, on the device)."""
         import torch
 
         self.width, self.height, self.num_gaussians = int(width), int(height), int(num_gaussians)
@@ -35,6 +39,8 @@ class SplatContext:
             st = self._lib.xad_splat_create(self.width, self.height, self.num_gaussians, int(pair_capacity_hint), ctypes.byref(handle))
         _lib.check(st, "xad_splat_create")
         self._handle = handle
+        if depth_mode != "checked":
+            self.set_depth_mode(depth_mode)
 
     def close(self):
         if getattr(self, "_handle", None):
@@ -51,6 +57,23 @@ class SplatContext:
         import torch
 
         return (stream if stream is not None else torch.cuda.current_stream(self.device)).cuda_stream
+
+    def set_depth_mode(self, mode):
+        _lib.check(self._lib.xad_splat_set_depth_mode(self._handle, DEPTH_MODES[mode] if isinstance(mode, str) else int(mode)),
+                   "xad_splat_set_depth_mode")
+
+    def lists(self):
+        """The tile lists of the last call: (range_begin, range_end, gaussians) as numpy uint32 arrays; tile t
+        (row-major) holds gaussians[range_begin[t]:range_end[t]] in compositing order.  Waits for the device."""
+        import numpy as np
+
+        tiles = ((self.width + 15) // 16) * ((self.height + 15) // 16)
+        begin, end = np.zeros(tiles, np.uint32), np.zeros(tiles, np.uint32)
+        pairs = self.stats()["pairs"]
+        ids = np.zeros(max(pairs, 1), np.uint32)
+        st = self._lib.xad_splat_get_lists(self._handle, begin.ctypes.data, end.ctypes.data, ids.ctypes.data, ids.size)
+        _lib.check(st, "xad_splat_get_lists")
+        return begin, end, ids[:pairs]
 
     def set_profiling(self, enabled):
         _lib.check(self._lib.xad_splat_set_profiling(self._handle, 1 if enabled else 0), "xad_splat_set_profiling")
