@@ -287,6 +287,21 @@ def splat_report(with_oracle, iters=30):
             entry["cpu_oracle"] = {"s_per_iter": cpu_s, "iters_per_s": 1.0 / cpu_s, "cores": oracle.max_threads(),
                                    "stage_s": ref["seconds"], "sample": "one full iteration"}
             entry["speedup_vs_cpu"] = cpu_s / per_iter
+            # The library's own templates on the host cores (xad_host_splat_step_f32: the per-pair graph of
+            # operation nodes, tiles dealt to threads), one full iteration with Adam in numpy.
+            cores = int(os.environ.get("OMP_NUM_THREADS", "0") or 0) or os.cpu_count()
+            splat.host_step(hp0[:, :64], hd[:64], ht[:16, :16], 16, 16, num_threads=cores)  # loads and warms the library
+            t0 = time.perf_counter()
+            host = splat.host_step(hp0, hd, ht, W, H, num_threads=cores)
+            hm2 = 0.1 * host["grads"]
+            hv2 = 0.001 * host["grads"] ** 2
+            stepped = hp0 - 1e-2 * (hm2 / 0.1) / (np.sqrt(hv2 / 0.001) + 1e-8)
+            host_s = time.perf_counter() - t0
+            entry["host_templates"] = {"s_per_iter": host_s, "iters_per_s": 1.0 / host_s, "cores": cores, "sample": "one full iteration",
+                                       "loss_matches_gpu": bool(abs(host["loss"] - first_loss) <= 1e-5 * first_loss),
+                                       "pairs": int(host["pairs"]),
+                                       "largest_parameter_change": float(np.abs(stepped - hp0).max())}
+            entry["speedup_vs_host_templates"] = host_s / per_iter
             entry["first_loss_matches_cpu"] = abs(first_loss - ref["loss"]) <= 1e-5 * ref["loss"]
             # Gradients of the first step against the fp64 oracle (binned with the fp32 projection's tile
             # rectangles), every one of the 9 x G against  1e-4 x mass + bound:  mass = the sum of the

@@ -209,6 +209,18 @@ int xad_splat_get_stats(xad_splat_context* ctx, uint64_t* pairs, uint32_t* longe
  * entries, at least the pair count.  Waits for the device. */
 int xad_splat_get_lists(xad_splat_context* ctx, uint32_t* range_begin, uint32_t* range_end,
                         uint32_t* gaussians, size_t capacity);
+/* The same step on the host cores, every pointer host memory: the CPU figure the
+ * GPU step is reported beside.  Tiles are dealt to num_threads threads (0: one per
+ * hardware thread); every (pixel, Gaussian) pair builds the renderer's per-pair
+ * graph from the library's nodes and runs its forward() and backward()
+ * (examples/mini-gaussian-splatting/gaussian_splatting_kernel.cu:42-55, :86-97),
+ * the parameters pass through the projection graph as on the GPU.  grads may be
+ * NULL (render and loss only); loss_out and pairs_out (number of (tile, Gaussian)
+ * pairs) may be NULL.  No entry of a list is skipped, so sums differ from the GPU
+ * step's by rounding and by terms with alpha below 1e-8. */
+int xad_host_splat_step_f32(int width, int height, int num_gaussians, const float* params,
+                            const float* depth, const float* target, float* image, float* grads,
+                            double* loss_out, uint64_t* pairs_out, int num_threads);
 
 /* Adam over structure-of-arrays parameters: `rows` rows of n floats each in
  * params, grads, m and v (device); row r uses row_learning_rates[r] (host).

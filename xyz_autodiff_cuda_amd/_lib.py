@@ -44,6 +44,7 @@ SIGNATURES = {
     "xad_splat_set_profiling": [_vp, _int],
     "xad_splat_set_depth_mode": [_vp, _int],
     "xad_splat_get_lists": [_vp, _vp, _vp, _vp, _sz],
+    "xad_host_splat_step_f32": [_int, _int, _int, _vp, _vp, _vp, _vp, _vp, ctypes.POINTER(ctypes.c_double), ctypes.POINTER(_u64), _int],
     "xad_splat_get_stats": [_vp, ctypes.POINTER(_u64), ctypes.POINTER(ctypes.c_uint32), ctypes.POINTER(_flt)],
     "xad_adam_step_f32": [_sz, _int, _vp, _vp, _vp, _vp, ctypes.POINTER(_flt), _flt, _flt, _flt, _int, _vp],
     "xad_training_config_defaults": [_vp],

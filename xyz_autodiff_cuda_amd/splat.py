@@ -125,6 +125,31 @@ class SplatContext:
         return out
 
 
+def host_step(params, depth, target, width, height, want_grads=True, num_threads=0):
+    """The step on the host cores (xad_host_splat_step_f32), numpy in and out: the CPU figure
+    the GPU step is reported beside.  params (9, G), depth (G,), target (height, width, 3), all
+    float32.  Returns a dict with image, grads (None unless wanted), loss and pairs."""
+    import numpy as np
+
+    params = np.ascontiguousarray(params, dtype=np.float32)
+    depth = np.ascontiguousarray(depth, dtype=np.float32)
+    target = np.ascontiguousarray(target, dtype=np.float32)
+    if params.ndim != 2 or params.shape[0] != len(PARAM_ROWS):
+        raise ValueError("params must have shape (9, G)")
+    G = params.shape[1]
+    if depth.shape != (G,) or target.shape != (height, width, 3):
+        raise ValueError("depth must have shape (G,) and target (height, width, 3)")
+    image = np.empty((height, width, 3), dtype=np.float32)
+    grads = np.empty_like(params) if want_grads else None
+    loss = ctypes.c_double(0.0)
+    pairs = ctypes.c_uint64(0)
+    st = _lib.load().xad_host_splat_step_f32(width, height, G, params.ctypes.data, depth.ctypes.data, target.ctypes.data,
+                                             image.ctypes.data, grads.ctypes.data if want_grads else None, ctypes.byref(loss),
+                                             ctypes.byref(pairs), int(num_threads))
+    _lib.check(st, "xad_host_splat_step_f32")
+    return {"image": image, "grads": grads, "loss": loss.value, "pairs": pairs.value}
+
+
 def adam_step(params, grads, m, v, learning_rates, iteration, beta1=0.9, beta2=0.999, eps=1e-8, stream=None):
     """In-place Adam over (rows, n) tensors; learning_rates: one float per row (or one float for all)."""
     import torch
