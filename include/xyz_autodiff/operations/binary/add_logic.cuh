@@ -29,8 +29,6 @@ struct AddLogic {
         XAD_UNROLL
         for (std::size_t i = 0; i < Dim; ++i) {
             const T g = out.grad(i);
-            const T l = lhs[i], r = rhs[i];
-            (void)l; (void)r;
             lhs.add_grad(i, g);
             rhs.add_grad(i, g);
         }

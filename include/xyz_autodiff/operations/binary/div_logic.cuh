@@ -30,7 +30,6 @@ struct DivLogic {
         for (std::size_t i = 0; i < Dim; ++i) {
             const T g = out.grad(i);
             const T l = lhs[i], r = rhs[i];
-            (void)l; (void)r;
             lhs.add_grad(i, g / r);
             rhs.add_grad(i, -g * l / (r * r));
         }

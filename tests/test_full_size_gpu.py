@@ -180,3 +180,19 @@ def test_splat_exactly_10k_gaussians_512(gpu, oracle):
 def test_splat_exactly_200k_gaussians_2048(gpu, oracle):
     figures = _splat_case(gpu, oracle, 200_000, 2048, 2048, (0.5, 40.0))
     assert 4_000_000 < figures["pairs"] < 12_000_000 and figures["longest_list"] < 5000
+
+
+@pytest.mark.parametrize("W,H,G,scale_px", [
+    (512, 400, 12_000, (1.0, 20.0)),    # 800 tiles: lists walked backward in eight pieces
+    (720, 720, 20_000, (1.0, 24.0)),    # 2025 tiles: four pieces
+    (1000, 1000, 40_000, (1.0, 24.0)),  # 3969 tiles: two pieces
+    (1100, 1100, 40_000, (1.0, 24.0)),  # 4761 tiles: one wavefront walks a tile's whole list
+])
+def test_splat_every_way_of_cutting_the_backward_walk(gpu, oracle, W, H, G, scale_px):
+    """The backward walk of a tile's list is cut into more pieces the fewer tiles an image has.  Every
+    such layout against the oracle, on scenes dense enough that lists span several pieces and many pixels
+    stop early (so that pieces start from a stored state, from the final state, or have nothing to do)."""
+    figures = _splat_case(gpu, oracle, G, W, H, scale_px)
+    tiles = ((W + 15) // 16) * ((H + 15) // 16)
+    assert figures["pairs"] / tiles > 64 and figures["longest_list"] > 128, figures
+

@@ -47,4 +47,11 @@ constexpr int kRecordGrads = 9;
 // Rows of the accumulator are 64 bytes apart, so the atomics on one Gaussian stay in one cache line.
 constexpr int kRecordGradStride = 16;
 
+// The loss is summed in kLossParts places, one cache line each (atomics on one address are taken one
+// after the other: a single sum would make every tile wait for all the others); the parameter
+// backward adds them up into element 0.  Part k is element kLossStride (1 + k).
+constexpr int kLossParts = 64;
+constexpr int kLossStride = 16;
+constexpr int kLossWords = kLossStride * (1 + kLossParts);
+
 }  // namespace xad_splat

@@ -50,9 +50,9 @@ __device__ __forceinline__ std::uint32_t read_lane(std::uint32_t v, int lane) {
 // Blocks take tickets, so a block only ever waits for blocks that are already running.  The state
 // words carry the launch's epoch, so nothing has to be cleared between launches: a word of another
 // epoch simply is not there yet.  data[n] receives the total.
-constexpr unsigned kScanBlock = 256;
-constexpr unsigned kScanItems = 8;
-constexpr unsigned kScanTile = kScanBlock * kScanItems;
+constexpr unsigned kScanBlock = 1024;
+constexpr unsigned kScanItems = 16;
+constexpr unsigned kScanTile = kScanBlock * kScanItems;  // few, large blocks: the chain of look-backs stays short
 
 __device__ __forceinline__ std::uint64_t scan_word(std::uint32_t epoch, std::uint32_t inclusive, std::uint32_t value) {
     return (static_cast<std::uint64_t>((epoch << 1) | inclusive) << 32) | value;
@@ -61,7 +61,7 @@ __device__ __forceinline__ std::uint64_t scan_word(std::uint32_t epoch, std::uin
 __global__ void __launch_bounds__(kScanBlock) scan_kernel(std::uint32_t* __restrict__ data, std::uint32_t n,
                                                           std::uint64_t* __restrict__ state, std::uint32_t* __restrict__ tickets,
                                                           std::uint32_t ticket_base, std::uint32_t epoch) {
-    __shared__ std::uint32_t shared[kScanBlock];
+    __shared__ std::uint32_t wave_total[kScanBlock / 64];
     __shared__ std::uint32_t block_index, block_exclusive;
     const unsigned t = threadIdx.x;
     if (t == 0) block_index = atomicAdd(tickets, 1u) - ticket_base;
@@ -71,9 +71,11 @@ __global__ void __launch_bounds__(kScanBlock) scan_kernel(std::uint32_t* __restr
 
     std::uint32_t v[kScanItems];
     if (first + kScanItems <= n) {
-        const uint4 lo = *reinterpret_cast<const uint4*>(data + first), hi = *reinterpret_cast<const uint4*>(data + first + 4);
-        v[0] = lo.x; v[1] = lo.y; v[2] = lo.z; v[3] = lo.w;
-        v[4] = hi.x; v[5] = hi.y; v[6] = hi.z; v[7] = hi.w;
+#pragma unroll
+        for (unsigned k = 0; k < kScanItems; k += 4) {
+            const uint4 q = *reinterpret_cast<const uint4*>(data + first + k);
+            v[k] = q.x; v[k + 1] = q.y; v[k + 2] = q.z; v[k + 3] = q.w;
+        }
     } else {
 #pragma unroll
         for (unsigned k = 0; k < kScanItems; ++k) v[k] = first + k < n ? data[first + k] : 0u;
@@ -82,17 +84,24 @@ __global__ void __launch_bounds__(kScanBlock) scan_kernel(std::uint32_t* __restr
 #pragma unroll
     for (unsigned k = 0; k < kScanItems; ++k) mine += v[k];
 
-    // inclusive scan of the 256 per-thread sums through LDS
-    shared[t] = mine;
-    __syncthreads();
-    for (unsigned step = 1; step < kScanBlock; step *= 2) {
-        const std::uint32_t other = t >= step ? shared[t - step] : 0u;
-        __syncthreads();
-        shared[t] += other;
-        __syncthreads();
+    // inclusive scan of the per-thread sums: within each wavefront by shuffles, across the wavefronts through LDS
+    const unsigned lane = t & 63u, wave = t >> 6;
+    std::uint32_t inclusive_in_wave = mine;
+#pragma unroll
+    for (unsigned step = 1; step < 64; step *= 2) {
+        const std::uint32_t other = __shfl_up(inclusive_in_wave, step, 64);
+        if (lane >= step) inclusive_in_wave += other;
     }
-    const std::uint32_t thread_exclusive = shared[t] - mine;
-    const std::uint32_t aggregate = shared[kScanBlock - 1];
+    if (lane == 63) wave_total[wave] = inclusive_in_wave;
+    __syncthreads();
+    std::uint32_t before_wave = 0, aggregate = 0;
+#pragma unroll
+    for (unsigned w = 0; w < kScanBlock / 64; ++w) {
+        const std::uint32_t total = wave_total[w];
+        before_wave += w < wave ? total : 0u;
+        aggregate += total;
+    }
+    const std::uint32_t thread_exclusive = before_wave + inclusive_in_wave - mine;
 
     // Look-back, by the block's first wavefront: 64 predecessors at a time, nearest first.  Each lane waits
     // for its predecessor's word of this epoch (that block holds an earlier ticket, so it is running),
@@ -126,14 +135,15 @@ __global__ void __launch_bounds__(kScanBlock) scan_kernel(std::uint32_t* __restr
 
     std::uint32_t running = block_exclusive + thread_exclusive;
     if (first + kScanItems <= n) {
-        std::uint32_t out[kScanItems];
 #pragma unroll
-        for (unsigned k = 0; k < kScanItems; ++k) {
-            out[k] = running;
-            running += v[k];
+        for (unsigned k = 0; k < kScanItems; k += 4) {
+            uint4 q;
+            q.x = running; running += v[k];
+            q.y = running; running += v[k + 1];
+            q.z = running; running += v[k + 2];
+            q.w = running; running += v[k + 3];
+            *reinterpret_cast<uint4*>(data + first + k) = q;
         }
-        *reinterpret_cast<uint4*>(data + first) = uint4{out[0], out[1], out[2], out[3]};
-        *reinterpret_cast<uint4*>(data + first + 4) = uint4{out[4], out[5], out[6], out[7]};
     } else {
 #pragma unroll
         for (unsigned k = 0; k < kScanItems; ++k) {

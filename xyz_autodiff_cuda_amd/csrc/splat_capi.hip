@@ -43,6 +43,8 @@ struct xad_splat_context {
     std::uint32_t *range_begin = nullptr, *range_end = nullptr;         // tiles each, adjacent
     float* final_T = nullptr;
     std::uint32_t* n_contrib = nullptr;
+    int segments = 1;                 // pieces a tile's list is cut into for the backward walk
+    float4* segment_state = nullptr;  // segments x pixels when segments > 1
     float* record_grads = nullptr;  // G x kRecordGradStride
     double* loss = nullptr;
     std::uint32_t* status = nullptr;  // kStatusWords
@@ -93,8 +95,9 @@ void carve_fixed(xad_splat_context* c, char* base, std::size_t* bytes) {
     c->range_end = c->range_begin ? c->range_begin + c->tiles : nullptr;
     c->final_T = k.take<float>(pixels);
     c->n_contrib = k.take<std::uint32_t>(pixels);
+    c->segment_state = c->segments > 1 ? k.take<float4>(pixels * static_cast<std::size_t>(c->segments)) : nullptr;
     c->record_grads = k.take<float>(G * kRecordGradStride);
-    c->loss = k.take<double>(1);
+    c->loss = k.take<double>(kLossWords);
     c->status = k.take<std::uint32_t>(kStatusWords);
     c->bin.tickets = k.take<std::uint32_t>(1);
     c->depth_sort_temp = k.take<char>(c->depth_sort_bytes ? c->depth_sort_bytes : 16);
@@ -293,6 +296,7 @@ extern "C" int xad_splat_create(int width, int height, int num_gaussians, std::s
     c->tiles_x = tiles_x;
     c->tiles_y = tiles_y;
     c->tiles = tiles_x * tiles_y;
+    c->segments = render_segments(width, height);
     c->depth_sort_bytes = depth_sort_temp_bytes(num_gaussians);
     int st = XAD_OK;
     std::size_t bytes = 0;
@@ -355,7 +359,7 @@ extern "C" int xad_splat_forward(xad_splat_context* c, const float* params, cons
     hipStream_t s = xad::as_stream(stream);
     if (int st = bin(c, params, depth, s)) return st;
     if (int st = launch_render_forward(s, c->width, c->height, c->range_begin, c->range_end, c->list, c->records, image,
-                                       c->final_T, c->n_contrib))
+                                       c->final_T, c->n_contrib, c->segments, c->segment_state))
         return st;
     mark(c, 3, s);
     collect_times(c, 3);
@@ -370,14 +374,15 @@ extern "C" int xad_splat_step(xad_splat_context* c, const float* params, const f
     for (int attempt = 0;; ++attempt) {
         if (int st = bin(c, params, depth, s)) return st;
         if (int st = launch_render_forward(s, c->width, c->height, c->range_begin, c->range_end, c->list, c->records, image,
-                                           c->final_T, c->n_contrib))
+                                           c->final_T, c->n_contrib, c->segments, c->segment_state))
             return st;
         mark(c, 3, s);
         if (int st = launch_render_backward(s, c->width, c->height, c->range_begin, c->range_end, c->list, c->records, image,
-                                            target, c->final_T, c->n_contrib, c->record_grads, c->loss))
+                                            target, c->final_T, c->n_contrib, c->record_grads, c->loss, c->segments,
+                                            c->segment_state))
             return st;
         mark(c, 4, s);
-        if (int st = launch_gaussian_backward(s, c->G, params, c->record_grads, grads)) return st;
+        if (int st = launch_gaussian_backward(s, c->G, params, c->record_grads, grads, c->loss)) return st;
         mark(c, 5, s);
         if (!loss_out) break;
         // the loss is read back, and with it what the device has to report

@@ -37,13 +37,13 @@ __global__ void __launch_bounds__(256) project_kernel(int G, const float* __rest
                                                       TileRect* __restrict__ rects_by_depth,
                                                       float* __restrict__ record_grads, double* __restrict__ loss) {
     const int g = blockIdx.x * 256 + threadIdx.x;
+    // what the compositing backward adds into starts from zero: the parts of the loss, this Gaussian's accumulator row
+    if (blockIdx.x == 0 && threadIdx.x < kLossParts) loss[kLossStride * (1 + threadIdx.x)] = 0.0;
     if (g >= G) return;
-    // what the compositing backward adds into starts from zero: this Gaussian's accumulator row, the loss
     {
         float4* row = reinterpret_cast<float4*>(record_grads + static_cast<std::size_t>(g) * kRecordGradStride);
 #pragma unroll
         for (int k = 0; k < kRecordGradStride / 4; ++k) row[k] = float4{0.f, 0.f, 0.f, 0.f};
-        if (g == 0) *loss = 0.0;
     }
     // the depth order of the previous call stays valid while every depth keeps its bits
     if (__builtin_bit_cast(std::uint32_t, depth[g]) != __builtin_bit_cast(std::uint32_t, ordered_depth[g]))
@@ -224,11 +224,26 @@ __device__ __forceinline__ std::uint32_t wave_max(std::uint32_t v) {
     return m01 > m23 ? m01 : m23;
 }
 
+// Small images have fewer tiles than the GPU has SIMDs, and a tile's backward walk is one long chain
+// of dependent instructions: a wavefront alone on its SIMD spends most of its time waiting for its own
+// results.  With kSplit the list of every tile is cut into `segments` pieces (whole groups of kPark
+// entries), each walked by a wavefront of its own in the backward pass.  For that the forward pass
+// leaves, per pixel and segment, the transmittance after the segment's last entry and the colour
+// composited behind it.  That colour is formed from the later segments' own sums (the colour sum is
+// restarted at every boundary), not as a difference of running totals, which would cancel.
+constexpr int kMaxSegments = 8;
+
+__device__ __forceinline__ std::uint32_t segment_length(std::uint32_t entries, int segments) {
+    const std::uint32_t groups = (entries + kPark - 1) / kPark;
+    return kPark * ((groups + static_cast<std::uint32_t>(segments) - 1) / static_cast<std::uint32_t>(segments));
+}
+
+template <bool kSplit>
 __global__ void __launch_bounds__(kChunk) render_forward_kernel(
     int width, int height, int tiles_x, int tiles, const std::uint32_t* __restrict__ range_begin,
     const std::uint32_t* __restrict__ range_end, const std::uint32_t* __restrict__ sorted_ids,
     const Record* __restrict__ records, float* __restrict__ image, float* __restrict__ final_T,
-    std::uint32_t* __restrict__ n_contrib) {
+    std::uint32_t* __restrict__ n_contrib, int segments, float4* __restrict__ segment_state) {
     __shared__ Staged staged[kChunk];
     const int tile = tile_of_block(blockIdx.x, tiles);
     if (tile >= tiles) return;
@@ -251,6 +266,21 @@ __global__ void __launch_bounds__(kChunk) render_forward_kernel(
         used[p] = 0;
     }
 
+    // kSplit: colour of the finished segments; red, green and blue hold the current segment's own
+    float done_red[kLanePixels], done_green[kLanePixels], done_blue[kLanePixels];
+#pragma unroll
+    for (int p = 0; p < kLanePixels; ++p) done_red[p] = done_green[p] = done_blue[p] = 0.f;
+    const std::uint32_t seg_len = kSplit ? segment_length(last - first, segments) : 0u;
+    std::uint32_t boundary = seg_len;
+    int segment = 0;
+    auto leave_segment_state = [&]() {
+#pragma unroll
+        for (int p = 0; p < kLanePixels; ++p)
+            if (x0 + p < width && y < height)
+                segment_state[(static_cast<std::size_t>(y) * width + x0 + p) * static_cast<std::size_t>(segments) + segment] =
+                    float4{T[p], red[p], green[p], blue[p]};  // the states of a pixel lie next to each other
+    };
+
     const float tile_x = static_cast<float>((tile % tiles_x) * kTile), tile_y = static_cast<float>((tile / tiles_x) * kTile);
     for (std::uint32_t base = first; base < last; base += kChunk) {
         __syncthreads();
@@ -264,6 +294,21 @@ __global__ void __launch_bounds__(kChunk) render_forward_kernel(
         // the staged entries that can be seen from this tile, front to back
         for (std::uint64_t todo = accumulate::wave::ballot(visible); todo != 0; todo &= todo - 1) {
             const int j = __builtin_ctzll(todo);
+            if constexpr (kSplit) {
+                // the first entry at or beyond a boundary closes the segments before it (the same for every lane)
+                while (base - first + j >= boundary) {
+                    leave_segment_state();
+#pragma unroll
+                    for (int p = 0; p < kLanePixels; ++p) {
+                        done_red[p] += red[p];
+                        done_green[p] += green[p];
+                        done_blue[p] += blue[p];
+                        red[p] = green[p] = blue[p] = 0.f;
+                    }
+                    ++segment;
+                    boundary += seg_len;
+                }
+            }
             const Staged r = staged[j];
             // exponent of the falloff as a polynomial in dx: (a_s dx + e) dx + f
             const float dy = py - r.cy;
@@ -289,6 +334,36 @@ __global__ void __launch_bounds__(kChunk) render_forward_kernel(
         const bool all_done = T[0] < kMinTransmittance && T[1] < kMinTransmittance && T[2] < kMinTransmittance &&
                               T[3] < kMinTransmittance;
         if (accumulate::wave::ballot(!all_done) == 0) break;
+    }
+    if constexpr (kSplit) {
+        leave_segment_state();  // of the segment the walk ended in
+#pragma unroll
+        for (int p = 0; p < kLanePixels; ++p) {
+            red[p] += done_red[p];
+            green[p] += done_green[p];
+            blue[p] += done_blue[p];
+        }
+        // What the backward walk of a segment needs is the colour behind it: the sum of the later segments'
+        // own colours.  Each state's colour is replaced by that sum (all loads first, then one pass).
+#pragma unroll
+        for (int p = 0; p < kLanePixels; ++p) {
+            if (x0 + p < width && y < height) {
+                float4* mine = segment_state + (static_cast<std::size_t>(y) * width + x0 + p) * static_cast<std::size_t>(segments);
+                float4 state[kMaxSegments];
+#pragma unroll
+                for (int k = 0; k < kMaxSegments; ++k) state[k] = mine[k < segment ? k : segment];
+                float behind[3] = {0.f, 0.f, 0.f};
+#pragma unroll
+                for (int k = kMaxSegments - 1; k >= 0; --k) {
+                    if (k <= segment) {  // the same for every lane
+                        mine[k] = float4{state[k].x, behind[0], behind[1], behind[2]};
+                        behind[0] += state[k].y;
+                        behind[1] += state[k].z;
+                        behind[2] += state[k].w;
+                    }
+                }
+            }
+        }
     }
 #pragma unroll
     for (int p = 0; p < kLanePixels; ++p) {
@@ -372,12 +447,13 @@ __device__ __forceinline__ float reduce_scatter9(const float (&v)[9], int lane) 
 // gradients are added to the global accumulator with consecutive lanes on
 // consecutive fields of consecutive entries: one atomic per (tile, Gaussian,
 // field), about seven accumulator rows (cache lines) per instruction.
+template <bool kSplit>
 __global__ void __launch_bounds__(kChunk) render_backward_kernel(
     int width, int height, int tiles_x, int tiles, const std::uint32_t* __restrict__ range_begin,
     const std::uint32_t* __restrict__ range_end, const std::uint32_t* __restrict__ sorted_ids,
     const Record* __restrict__ records, const float* __restrict__ image, const float* __restrict__ target,
     const float* __restrict__ final_T, const std::uint32_t* __restrict__ n_contrib, float* __restrict__ record_grads,
-    double* __restrict__ loss) {
+    double* __restrict__ loss, int segments, const float4* __restrict__ segment_state) {
     __shared__ Staged staged[kChunk];
     __shared__ std::uint32_t staged_id[kChunk];
     // Row sums wait here until a group of kPark list entries is complete.  Small on purpose: LDS per
@@ -385,7 +461,11 @@ __global__ void __launch_bounds__(kChunk) render_backward_kernel(
     __shared__ float parked[kPark][4][9];  // [list entry within its group][row of 16 lanes][value]
     __shared__ int parked_entry[kPark];    // which staged entry that is
 
-    const int tile = tile_of_block(blockIdx.x, tiles);
+    // kSplit: all tiles' first segments, then all second ones, ...: every XCD gets its band of tiles of every
+    // segment (the late segments are the ones that often have nothing to walk)
+    const unsigned blocks_per_segment = kSplit ? gridDim.x / static_cast<unsigned>(segments) : gridDim.x;
+    const int segment = kSplit ? static_cast<int>(blockIdx.x / blocks_per_segment) : 0;
+    const int tile = tile_of_block(static_cast<int>(blockIdx.x % blocks_per_segment), tiles);
     if (tile >= tiles) return;
     const int lane = threadIdx.x;
     const int x0 = (tile % tiles_x) * kTile + (lane & 3) * kLanePixels;
@@ -419,22 +499,49 @@ __global__ void __launch_bounds__(kChunk) render_backward_kernel(
             my_max = used[p] > my_max ? used[p] : my_max;
         }
     }
-    {
+    if (segment == 0) {
         const float tile_loss = accumulate::wave::sum(my_loss);
-        if (lane == 0 && tile_loss != 0.f) detail::atomic_add(loss, static_cast<double>(tile_loss));
+        if (lane == 0 && tile_loss != 0.f)
+            detail::atomic_add(loss + kLossStride * (1 + tile % kLossParts), static_cast<double>(tile_loss));
     }
     const std::uint32_t deepest = wave_max(my_max);  // entries [0, deepest) were composited by some pixel
     if (deepest == 0) return;
     const std::uint32_t first = range_begin[tile];
     const float px0 = static_cast<float>(x0);
+    // this block walks entries [walk_first, walk_last) of the list, back to front
+    std::uint32_t walk_first = 0, walk_last = deepest;
+    if constexpr (kSplit) {
+        const std::uint32_t seg_len = segment_length(range_end[tile] - first, segments);
+        walk_first = static_cast<std::uint32_t>(segment) * seg_len;
+        if (walk_first >= deepest) return;
+        walk_last = walk_first + seg_len < deepest ? walk_first + seg_len : deepest;
+        // A pixel that went on beyond this segment starts from what the forward pass left for the
+        // segment's end: the transmittance there, and the colour composited behind it.
+#pragma unroll
+        for (int p = 0; p < kLanePixels; ++p) {
+            if (used[p] > walk_last) {
+                // the states of a pixel lie next to each other
+                const float4* mine = segment_state + (static_cast<std::size_t>(y) * width + x0 + p) * static_cast<std::size_t>(segments);
+                const float4 state = mine[segment];
+                T[p] = state.x;
+                const float behind[3] = {state.y, state.z, state.w};
+                D[p] = -::fmaf(dC[p][2], behind[2], ::fmaf(dC[p][1], behind[1], dC[p][0] * behind[0]));
+            }
+        }
+    }
+    // What has been loaded so far is first needed inside the loop over the entries.  Left to itself the
+    // wait for those loads ends up there, where it also waits, at every entry, for the atomics issued
+    // since; a use of the values here settles them before the loop.
+#pragma unroll
+    for (int p = 0; p < kLanePixels; ++p) asm volatile("" : "+v"(T[p]), "+v"(D[p]));
     // which of the nine row sums this lane ends up with; eight lanes and one more per row park theirs
     const int park_index = reduced_index(lane);
     const bool parks = !(lane & 2) || (lane & 15) == 2;
 
     const float tile_x = static_cast<float>((tile % tiles_x) * kTile), tile_y = static_cast<float>((tile / tiles_x) * kTile);
-    for (std::uint32_t chunk = (deepest + kChunk - 1) / kChunk; chunk-- > 0;) {
-        const std::uint32_t chunk_first = chunk * kChunk;
-        const int count = static_cast<int>(deepest - chunk_first < kChunk ? deepest - chunk_first : kChunk);
+    for (std::uint32_t chunk = (walk_last - walk_first + kChunk - 1) / kChunk; chunk-- > 0;) {
+        const std::uint32_t chunk_first = walk_first + chunk * kChunk;
+        const int count = static_cast<int>(walk_last - chunk_first < kChunk ? walk_last - chunk_first : kChunk);
         __syncthreads();
         bool visible = false;
         if (lane < count) {
@@ -541,9 +648,15 @@ __global__ void __launch_bounds__(kChunk) render_backward_kernel(
 // straight through.
 __global__ void __launch_bounds__(256) gaussian_backward_kernel(int G, const float* __restrict__ params,
                                                                 const float* __restrict__ record_grads,
-                                                                float* __restrict__ grads) {
+                                                                float* __restrict__ grads, double* __restrict__ loss) {
     const int g = blockIdx.x * 256 + threadIdx.x;
     if (g >= G) return;
+    if (g == 0) {
+        double total = 0.0;
+#pragma unroll 8
+        for (int k = 0; k < kLossParts; ++k) total += loss[kLossStride * (1 + k)];
+        loss[0] = total;
+    }
     const std::size_t n = static_cast<std::size_t>(G);
     const float* acc = record_grads + static_cast<std::size_t>(g) * kRecordGradStride;
 
@@ -603,12 +716,23 @@ int launch_depth_keys(hipStream_t s, int G, const float* depth, std::uint32_t* k
 
 static unsigned padded_tile_blocks(int tiles) { return static_cast<unsigned>(((tiles + 7) / 8) * 8); }
 
+int render_segments(int width, int height) {
+    const int tiles = ((width + kTile - 1) / kTile) * ((height + kTile - 1) / kTile);
+    return tiles <= 1024 ? 8 : (tiles <= 2048 ? 4 : (tiles <= 4096 ? 2 : 1));
+}
+
 int launch_render_forward(hipStream_t s, int width, int height, const std::uint32_t* range_begin,
                           const std::uint32_t* range_end, const std::uint32_t* sorted_ids, const Record* records,
-                          float* image, float* final_T, std::uint32_t* n_contrib) {
+                          float* image, float* final_T, std::uint32_t* n_contrib, int segments, float4* segment_state) {
     const int tiles_x = (width + kTile - 1) / kTile, tiles = tiles_x * ((height + kTile - 1) / kTile);
-    hipLaunchKernelGGL(render_forward_kernel, dim3(padded_tile_blocks(tiles)), dim3(kChunk), 0, s, width, height,
-                       tiles_x, tiles, range_begin, range_end, sorted_ids, records, image, final_T, n_contrib);
+    XAD_REQUIRE(segments >= 1 && (segments == 1 || segment_state), "splat: a split walk needs its per-segment state");
+    if (segments > 1)
+        hipLaunchKernelGGL(render_forward_kernel<true>, dim3(padded_tile_blocks(tiles)), dim3(kChunk), 0, s, width, height,
+                           tiles_x, tiles, range_begin, range_end, sorted_ids, records, image, final_T, n_contrib, segments,
+                           segment_state);
+    else
+        hipLaunchKernelGGL(render_forward_kernel<false>, dim3(padded_tile_blocks(tiles)), dim3(kChunk), 0, s, width, height,
+                           tiles_x, tiles, range_begin, range_end, sorted_ids, records, image, final_T, n_contrib, 1, nullptr);
     XAD_HIP_TRY(hipGetLastError());
     return XAD_OK;
 }
@@ -616,18 +740,26 @@ int launch_render_forward(hipStream_t s, int width, int height, const std::uint3
 int launch_render_backward(hipStream_t s, int width, int height, const std::uint32_t* range_begin,
                            const std::uint32_t* range_end, const std::uint32_t* sorted_ids, const Record* records,
                            const float* image, const float* target, const float* final_T,
-                           const std::uint32_t* n_contrib, float* record_grads, double* loss) {
+                           const std::uint32_t* n_contrib, float* record_grads, double* loss, int segments,
+                           const float4* segment_state) {
     const int tiles_x = (width + kTile - 1) / kTile, tiles = tiles_x * ((height + kTile - 1) / kTile);
-    hipLaunchKernelGGL(render_backward_kernel, dim3(padded_tile_blocks(tiles)), dim3(kChunk), 0, s, width, height,
-                       tiles_x, tiles, range_begin, range_end, sorted_ids, records, image, target, final_T, n_contrib,
-                       record_grads, loss);
+    XAD_REQUIRE(segments >= 1 && segments <= kMaxSegments && (segments == 1 || segment_state),
+                "splat: a split walk takes up to %d segments and needs its per-segment state", kMaxSegments);
+    if (segments > 1)
+        hipLaunchKernelGGL(render_backward_kernel<true>, dim3(padded_tile_blocks(tiles) * static_cast<unsigned>(segments)),
+                           dim3(kChunk), 0, s, width, height, tiles_x, tiles, range_begin, range_end, sorted_ids, records, image,
+                           target, final_T, n_contrib, record_grads, loss, segments, segment_state);
+    else
+        hipLaunchKernelGGL(render_backward_kernel<false>, dim3(padded_tile_blocks(tiles)), dim3(kChunk), 0, s, width, height,
+                           tiles_x, tiles, range_begin, range_end, sorted_ids, records, image, target, final_T, n_contrib,
+                           record_grads, loss, 1, nullptr);
     XAD_HIP_TRY(hipGetLastError());
     return XAD_OK;
 }
 
-int launch_gaussian_backward(hipStream_t s, int G, const float* params, const float* record_grads, float* grads) {
+int launch_gaussian_backward(hipStream_t s, int G, const float* params, const float* record_grads, float* grads, double* loss) {
     hipLaunchKernelGGL(gaussian_backward_kernel, dim3(xad::blocks_for(G, 256)), dim3(256), 0, s, G, params, record_grads,
-                       grads);
+                       grads, loss);
     XAD_HIP_TRY(hipGetLastError());
     return XAD_OK;
 }

@@ -67,12 +67,17 @@ int launch_binning(hipStream_t s, const BinPlan& p, const std::uint32_t* by_dept
                    bool clear_depth_flag);
 int launch_render_forward(hipStream_t s, int width, int height, const std::uint32_t* range_begin,
                           const std::uint32_t* range_end, const std::uint32_t* sorted_ids, const Record* records,
-                          float* image, float* final_T, std::uint32_t* n_contrib);
+                          float* image, float* final_T, std::uint32_t* n_contrib, int segments, float4* segment_state);
 int launch_render_backward(hipStream_t s, int width, int height, const std::uint32_t* range_begin,
                            const std::uint32_t* range_end, const std::uint32_t* sorted_ids, const Record* records,
                            const float* image, const float* target, const float* final_T,
-                           const std::uint32_t* n_contrib, float* record_grads, double* loss);
-int launch_gaussian_backward(hipStream_t s, int G, const float* params, const float* record_grads, float* grads);
+                           const std::uint32_t* n_contrib, float* record_grads, double* loss, int segments,
+                           const float4* segment_state);
+// Pieces a tile's list is cut into for the backward walk (1, 2, 4 or 8: more for images with few tiles);
+// segment_state holds that many float4 per pixel when it is more than one.
+int render_segments(int width, int height);
+// Also adds the parts of the loss up into loss[0].
+int launch_gaussian_backward(hipStream_t s, int G, const float* params, const float* record_grads, float* grads, double* loss);
 
 // The stable radix sort of (depth bits, index) that yields the depth order (rocPRIM; runs only when a depth changed).
 std::size_t depth_sort_temp_bytes(int G);
