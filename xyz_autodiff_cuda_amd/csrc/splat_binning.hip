@@ -154,8 +154,122 @@ __global__ void __launch_bounds__(kScanBlock) scan_kernel(std::uint32_t* __restr
 }
 
 // ---------------------------------------------------------------------------
-// Level A.  One wavefront per block; block = (range of Gaussians) x (group of 64 supertiles), blocks of
-// one range adjacent so that they read the same rectangles from the same L2.
+// Transpose of a 64 x 64 bit matrix held one row per lane (lo = columns 0..31, hi = columns 32..63):
+// afterwards lane t holds column t, bit j of it being bit t of lane j's row.  The usual recursive block
+// swap: at distance k, the lanes whose bit k is clear keep their columns with bit k clear and receive,
+// into their columns with bit k set, the partner's columns with bit k clear; the others the reverse.
+__device__ __forceinline__ void transpose_64x64(std::uint32_t& lo, std::uint32_t& hi, int lane) {
+    {
+        const std::uint32_t other_lo = __shfl_xor(lo, 32, 64), other_hi = __shfl_xor(hi, 32, 64);
+        if (lane & 32)
+            lo = other_hi;
+        else
+            hi = other_lo;
+    }
+    constexpr std::uint32_t kClear[5] = {0x0000ffffu, 0x00ff00ffu, 0x0f0f0f0fu, 0x33333333u, 0x55555555u};
+#pragma unroll
+    for (int step = 0; step < 5; ++step) {
+        const int k = 16 >> step;
+        const std::uint32_t m = kClear[step];
+        const std::uint32_t other_lo = __shfl_xor(lo, k, 64), other_hi = __shfl_xor(hi, k, 64);
+        if (lane & k) {
+            lo = ((other_lo >> k) & m) | (lo & ~m);
+            hi = ((other_hi >> k) & m) | (hi & ~m);
+        } else {
+            lo = (lo & m) | ((other_lo & m) << k);
+            hi = (hi & m) | ((other_hi & m) << k);
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Both levels turn 64 rectangles into 64 lists the same way.  Lane = rectangle: the 8 x 8 cells it covers,
+// as a 64-bit mask (cell = 8 row + column).  After the transpose, lane = cell, and the mask says which of
+// the 64 rectangles cover it: its population count is the cell's count, its set bits, from the lowest, are
+// the cell's members in order.
+
+// Bits x0..x1 of every row y0..y1 (all within 0..7; empty if a range is).
+__device__ __forceinline__ std::uint64_t block_mask(int x0, int x1, int y0, int y1) {
+    if (x0 > x1 || y0 > y1) return 0;
+    const std::uint64_t row = ((std::uint64_t(1) << (x1 - x0 + 1)) - 1) << x0;
+    const std::uint64_t rows = (0x0101010101010101ull >> (8 * (7 - (y1 - y0)))) << (8 * y0);
+    return row * rows;  // the multiplier has one bit per row: no carries
+}
+
+// Writes the members of every lane's mask (lane j's value `id` for bit j) to out[from ...], lane by lane.
+// One entry per lane and turn would scatter every store over 64 cache lines.  The entries go through LDS
+// instead: lane t puts its run at [before, before + count) there, and the runs are written out with
+// consecutive lanes on consecutive entries of a run (a window of LDS at a time).  Stores at or beyond
+// `capacity` are dropped.  Returns the lane's count.  Every lane of the wavefront must call it.
+constexpr std::uint32_t kStageEntries = 1024;
+struct RunStage {
+    std::uint32_t staged[kStageEntries];
+    std::uint32_t run_begin[65];
+    std::uint32_t run_dest[64];
+};
+
+__device__ __forceinline__ std::uint32_t write_runs(RunStage& lds, std::uint64_t mine, std::uint32_t id, std::uint32_t from,
+                                                    std::uint32_t* __restrict__ out, std::uint32_t capacity, int lane) {
+    const std::uint32_t count = static_cast<std::uint32_t>(__builtin_popcountll(mine));
+    std::uint32_t inclusive = count;
+#pragma unroll
+    for (int step = 1; step < 64; step *= 2) {
+        const std::uint32_t other = __shfl_up(inclusive, step, 64);
+        if (lane >= step) inclusive += other;
+    }
+    const std::uint32_t total = read_lane(inclusive, 63);
+    std::uint32_t next = inclusive - count;  // where this lane's next entry goes
+    __syncthreads();                         // the previous call's readers are done
+    lds.run_begin[lane] = next;
+    if (lane == 63) lds.run_begin[64] = total;
+    lds.run_dest[lane] = from;
+    for (std::uint32_t window = 0; window < total; window += kStageEntries) {
+        // every lane stays in the loop until the last one is done: the exchange below reads other lanes' registers
+        while (ballot(mine != 0 && next < window + kStageEntries) != 0) {
+            const bool has = mine != 0 && next < window + kStageEntries;
+            const int j = has ? __builtin_ctzll(mine) : 0;
+            const std::uint32_t member = __shfl(id, j, 64);
+            if (has) {
+                lds.staged[next - window] = member;
+                ++next;
+                mine &= mine - 1;
+            }
+        }
+        __syncthreads();
+        const std::uint32_t end = total - window < kStageEntries ? total - window : kStageEntries;
+        for (std::uint32_t e = static_cast<std::uint32_t>(lane); e < end; e += 64) {
+            const std::uint32_t at = window + e;
+            int t = 0;  // the run `at` lies in: the last one that begins at or before it (empty runs begin where the next one does)
+#pragma unroll
+            for (int step = 32; step > 0; step >>= 1)
+                if (lds.run_begin[t + step] <= at) t += step;
+            const std::uint32_t dest = lds.run_dest[t] + (at - lds.run_begin[t]);
+            if (dest < capacity) out[dest] = lds.staged[e];
+        }
+        __syncthreads();
+    }
+    return count;
+}
+
+// Supertiles are numbered group by group, a group being 8 x 8 supertiles (row-major within the group,
+// groups row-major over the image); numbers whose supertile lies beyond the image stay empty.
+struct SuperCoords {
+    int x, y;
+    bool inside;
+};
+__device__ __forceinline__ SuperCoords super_coords(const BinPlan& p, int s) {
+    const int group = s >> 6, local = s & 63;
+    SuperCoords c;
+    c.x = (group % p.group_x) * 8 + (local & 7);
+    c.y = (group / p.group_x) * 8 + (local >> 3);
+    c.inside = c.x < p.super_x && c.y < p.super_y;
+    return c;
+}
+
+// ---------------------------------------------------------------------------
+// Level A.  One wavefront per block; block = (range of Gaussians) x (group of 8 x 8 supertiles), blocks of
+// one range adjacent so that they read the same rectangles from the same L2.  64 Gaussians at a time:
+// lane = Gaussian, mask = the group's supertiles its rectangle reaches; transposed, lane = supertile.
 // kFill = false: matrix_a[supertile * ranges_a + range] = number of Gaussians of the range that
 // touch the supertile.  kFill = true: matrix_a holds the scanned counts; the Gaussians are written.
 // rects_by_depth[i] is the rectangle of Gaussian by_depth[i]: both loads of a lane are independent and coalesced.
@@ -163,54 +277,40 @@ template <bool kFill>
 __global__ void __launch_bounds__(64) super_kernel(BinPlan p, const std::uint32_t* __restrict__ by_depth,
                                                    const TileRect* __restrict__ rects_by_depth,
                                                    std::uint32_t* __restrict__ matrix_a, std::uint32_t* __restrict__ list_a) {
+    __shared__ RunStage stage;
     const int lane = static_cast<int>(threadIdx.x);
     const int group = static_cast<int>(blockIdx.x % static_cast<unsigned>(p.groups));
     const int range = static_cast<int>(blockIdx.x / static_cast<unsigned>(p.groups));
-    const int s = group * 64 + lane;
-    const bool owner = s < p.supers;
-    const int sx = s % p.super_x, sy = s / p.super_x;
-    // rows of supertiles this group reaches into
-    const int last_super = group * 64 + 63 < p.supers - 1 ? group * 64 + 63 : p.supers - 1;
-    const int row_lo = (group * 64) / p.super_x, row_hi = last_super / p.super_x;
-    const std::size_t cell = static_cast<std::size_t>(owner ? s : 0) * p.ranges_a + range;
-    std::uint32_t cursor = (kFill && owner) ? matrix_a[cell] : 0u;
+    const int origin_x = (group % p.group_x) * 8, origin_y = (group / p.group_x) * 8;  // in supertiles
+    const std::size_t cell = static_cast<std::size_t>(group * 64 + lane) * p.ranges_a + range;
+    std::uint32_t cursor = kFill ? matrix_a[cell] : 0u;
     std::uint32_t count = 0;
 
     const int first = range * p.range_a;
     const int last = first + p.range_a < p.G ? first + p.range_a : p.G;
     for (int base = first; base < last; base += 64) {
         const int i = base + lane;
-        std::uint32_t g = 0, lo = 0, hi = 0;
-        bool candidate = false;
+        std::uint32_t g = 0;
+        std::uint64_t mask = 0;
         if (i < last) {
             g = by_depth[i];
             const TileRect rc = rects_by_depth[i];
             if (rc.x0 <= rc.x1) {
-                const int y0 = rc.y0 >> 3, y1 = rc.y1 >> 3;
-                candidate = y1 >= row_lo && y0 <= row_hi;
-                lo = static_cast<std::uint32_t>(rc.x0 >> 3) | (static_cast<std::uint32_t>(y0) << 16);
-                hi = static_cast<std::uint32_t>(rc.x1 >> 3) | (static_cast<std::uint32_t>(y1) << 16);
+                const int x0 = (rc.x0 >> 3) - origin_x, x1 = (rc.x1 >> 3) - origin_x;
+                const int y0 = (rc.y0 >> 3) - origin_y, y1 = (rc.y1 >> 3) - origin_y;
+                mask = block_mask(x0 > 0 ? x0 : 0, x1 < 7 ? x1 : 7, y0 > 0 ? y0 : 0, y1 < 7 ? y1 : 7);
             }
         }
-        for (std::uint64_t todo = ballot(candidate); todo != 0; todo &= todo - 1) {
-            const int j = __builtin_ctzll(todo);
-            const std::uint32_t l = read_lane(lo, j), h = read_lane(hi, j), gj = read_lane(g, j);
-            const int x0 = static_cast<int>(l & 0xffffu), y0 = static_cast<int>(l >> 16);
-            const int x1 = static_cast<int>(h & 0xffffu), y1 = static_cast<int>(h >> 16);
-            const bool covered = owner && sx >= x0 && sx <= x1 && sy >= y0 && sy <= y1;
-            if constexpr (kFill) {
-                if (covered) {
-                    if (cursor < p.capacity_a) list_a[cursor] = gj;
-                    ++cursor;
-                }
-            } else {
-                count += covered ? 1u : 0u;
-            }
+        std::uint32_t lo = static_cast<std::uint32_t>(mask), hi = static_cast<std::uint32_t>(mask >> 32);
+        transpose_64x64(lo, hi, lane);  // now: which of the 64 Gaussians reach this lane's supertile
+        const std::uint64_t mine = (static_cast<std::uint64_t>(hi) << 32) | lo;
+        if constexpr (kFill) {
+            cursor += write_runs(stage, mine, g, cursor, list_a, p.capacity_a, lane);
+        } else {
+            count += static_cast<std::uint32_t>(__builtin_popcountll(mine));
         }
     }
-    if constexpr (!kFill) {
-        if (owner) matrix_a[cell] = count;
-    }
+    if constexpr (!kFill) matrix_a[cell] = count;
 }
 
 // ---------------------------------------------------------------------------
@@ -233,7 +333,7 @@ __global__ void __launch_bounds__(256) plan_kernel(BinPlan p, const std::uint32_
     for (int base = 0; base < p.supers; base += 256) {
         const int s = base + static_cast<int>(t);
         std::uint32_t waves = 0;
-        if (s < p.supers) {
+        if (s < p.supers && super_coords(p, s).inside) {
             std::uint32_t begin = offsets_a[static_cast<std::size_t>(s) * p.ranges_a];
             std::uint32_t end = offsets_a[static_cast<std::size_t>(s + 1) * p.ranges_a];
             begin = begin < p.capacity_a ? begin : p.capacity_a;
@@ -268,35 +368,6 @@ __global__ void __launch_bounds__(256) plan_kernel(BinPlan p, const std::uint32_
 }
 
 // ---------------------------------------------------------------------------
-// Transpose of a 64 x 64 bit matrix held one row per lane (lo = columns 0..31, hi = columns 32..63):
-// afterwards lane t holds column t, bit j of it being bit t of lane j's row.  The usual recursive block
-// swap: at distance k, the lanes whose bit k is clear keep their columns with bit k clear and receive,
-// into their columns with bit k set, the partner's columns with bit k clear; the others the reverse.
-__device__ __forceinline__ void transpose_64x64(std::uint32_t& lo, std::uint32_t& hi, int lane) {
-    {
-        const std::uint32_t other_lo = __shfl_xor(lo, 32, 64), other_hi = __shfl_xor(hi, 32, 64);
-        if (lane & 32)
-            lo = other_hi;
-        else
-            hi = other_lo;
-    }
-    constexpr std::uint32_t kClear[5] = {0x0000ffffu, 0x00ff00ffu, 0x0f0f0f0fu, 0x33333333u, 0x55555555u};
-#pragma unroll
-    for (int step = 0; step < 5; ++step) {
-        const int k = 16 >> step;
-        const std::uint32_t m = kClear[step];
-        const std::uint32_t other_lo = __shfl_xor(lo, k, 64), other_hi = __shfl_xor(hi, k, 64);
-        if (lane & k) {
-            lo = ((other_lo >> k) & m) | (lo & ~m);
-            hi = ((other_hi >> k) & m) | (hi & ~m);
-        } else {
-            lo = (lo & m) | ((other_lo & m) << k);
-            hi = (hi & m) | ((other_hi & m) << k);
-        }
-    }
-}
-
-// ---------------------------------------------------------------------------
 // Level B.  One wavefront per block: wavefront w serves entries [64 q, 64 q + 64) of the list of supertile s,
 // where first_wave[s] <= w < first_wave[s + 1] and q = w - first_wave[s]; after the transpose, lane = tile of
 // the supertile (row-major, 8 per row).  The counts of supertile s live at
@@ -311,6 +382,7 @@ __global__ void __launch_bounds__(64) tile_kernel(BinPlan p, const std::uint32_t
                                                   std::uint32_t* __restrict__ matrix_b, std::uint32_t* __restrict__ list,
                                                   std::uint32_t* __restrict__ range_begin, std::uint32_t* __restrict__ range_end,
                                                   std::uint32_t* __restrict__ status) {
+    __shared__ RunStage stage;
     const int lane = static_cast<int>(threadIdx.x);
     const std::uint32_t w = blockIdx.x;
     const std::uint32_t used = first_wave[p.supers];
@@ -334,21 +406,16 @@ __global__ void __launch_bounds__(64) tile_kernel(BinPlan p, const std::uint32_t
     end = end < p.capacity_a ? end : p.capacity_a;
     const std::uint32_t i = begin + q * kBinRangeB + static_cast<std::uint32_t>(lane);
 
-    const int base_x = (s % p.super_x) * 8, base_y = (s / p.super_x) * 8;
+    const SuperCoords where = super_coords(p, s);
+    const int base_x = where.x * 8, base_y = where.y * 8;
     std::uint32_t g = 0, mask_lo = 0, mask_hi = 0;
     if (i < end) {
         g = list_a[i];
         const TileRect rc = rects[g];
-        const int x0 = rc.x0 - base_x > 0 ? rc.x0 - base_x : 0, x1 = rc.x1 - base_x < 7 ? rc.x1 - base_x : 7;
-        const int y0 = rc.y0 - base_y > 0 ? rc.y0 - base_y : 0, y1 = rc.y1 - base_y < 7 ? rc.y1 - base_y : 7;
-        if (x0 <= x1 && y0 <= y1) {
-            // bits x0..x1 of a row, repeated in rows y0..y1 (the multiplier has one bit per row: no carries)
-            const std::uint64_t row = ((std::uint64_t(1) << (x1 - x0 + 1)) - 1) << x0;
-            const std::uint64_t rows = (0x0101010101010101ull >> (8 * (7 - (y1 - y0)))) << (8 * y0);
-            const std::uint64_t mask = row * rows;
-            mask_lo = static_cast<std::uint32_t>(mask);
-            mask_hi = static_cast<std::uint32_t>(mask >> 32);
-        }
+        const std::uint64_t mask = block_mask(rc.x0 - base_x > 0 ? rc.x0 - base_x : 0, rc.x1 - base_x < 7 ? rc.x1 - base_x : 7,
+                                              rc.y0 - base_y > 0 ? rc.y0 - base_y : 0, rc.y1 - base_y < 7 ? rc.y1 - base_y : 7);
+        mask_lo = static_cast<std::uint32_t>(mask);
+        mask_hi = static_cast<std::uint32_t>(mask >> 32);
     }
     transpose_64x64(mask_lo, mask_hi, lane);  // now: which of the 64 entries cover this lane's tile
     const int tx = base_x + (lane & 7), ty = base_y + (lane >> 3);
@@ -359,19 +426,8 @@ __global__ void __launch_bounds__(64) tile_kernel(BinPlan p, const std::uint32_t
     if constexpr (!kFill) {
         matrix_b[cell] = static_cast<std::uint32_t>(__builtin_popcountll(mine));
     } else {
-        std::uint32_t cursor = matrix_b[cell];
-        const std::uint32_t from = cursor;
-        // every lane stays in the loop until the last one is done: the exchange below reads other lanes' registers
-        while (ballot(mine != 0) != 0) {
-            const bool has = mine != 0;
-            const int j = has ? __builtin_ctzll(mine) : 0;
-            const std::uint32_t gj = __shfl(g, j, 64);
-            if (has) {
-                if (cursor < p.capacity) list[cursor] = gj;
-                ++cursor;
-                mine &= mine - 1;
-            }
-        }
+        const std::uint32_t from = matrix_b[cell];
+        write_runs(stage, mine, g, from, list, p.capacity, lane);
         if (q == 0 && owner) {
             // this tile's list: from the first cell of the tile to the first cell of the next one
             const std::size_t next_cell = static_cast<std::size_t>(wave0) * 64 + static_cast<std::size_t>(lane + 1) * waves;
@@ -400,8 +456,9 @@ BinPlan make_bin_plan(int G, int tiles_x, int tiles_y, std::uint32_t capacity, s
     p.tiles_y = tiles_y;
     p.super_x = (tiles_x + 7) / 8;
     p.super_y = (tiles_y + 7) / 8;
-    p.supers = p.super_x * p.super_y;
-    p.groups = (p.supers + 63) / 64;
+    p.group_x = (p.super_x + 7) / 8;
+    p.groups = p.group_x * ((p.super_y + 7) / 8);
+    p.supers = p.groups * 64;  // numbered group by group; those beyond the image stay empty
     // about 8192 wavefronts at level A (short ones: a wavefront's chunks of 64 Gaussians are a chain of memory
     // latencies), and never less than 64 Gaussians per wavefront
     const long long per_wave = (static_cast<long long>(G) * p.groups + 8191) / 8192;

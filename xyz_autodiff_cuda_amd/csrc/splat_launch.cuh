@@ -35,8 +35,9 @@ int launch_depth_rank(hipStream_t s, int G, const std::uint32_t* by_depth, std::
 constexpr std::uint32_t kBinRangeB = 64;  // list entries a wavefront handles at level B: one per lane
 struct BinPlan {
     int G, tiles_x, tiles_y;
-    int super_x, super_y, supers;  // supertiles of 8 x 8 tiles
-    int groups;                    // groups of 64 supertiles
+    int super_x, super_y;          // supertiles of 8 x 8 tiles across and down the image
+    int group_x, groups;           // groups of 8 x 8 supertiles: across the image, and in all
+    int supers;                    // supertile numbers: 64 per group, whether inside the image or not
     int range_a, ranges_a;         // Gaussians per wavefront at level A, and how many such ranges
     std::uint32_t capacity;        // (tile, Gaussian) pairs the lists can hold
     std::uint32_t capacity_a;      // (supertile, Gaussian) pairs level A may produce: at most capacity (the buffer's size)
