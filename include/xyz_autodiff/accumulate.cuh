@@ -186,7 +186,8 @@ public:
     // row are not sent to `global` lane by lane (Width instructions, each touching up to 64 rows) but
     // are first gathered per wavefront in `staging` (spill_bytes(blockDim.x) bytes of LDS, 4-byte
     // aligned), kStageRows at a time, and written out with consecutive lanes on consecutive elements
-    // of consecutive rows, which cuts the number of memory requests several times.  Must be called
+    // of consecutive rows, which cuts the number of memory requests several times.  Rows wait there
+    // until kStageRows have come together; flush() writes out what is left.  Must be called
     // before the first add(); add() must then be reached by all lanes of a wavefront together
     // whatever the strategy.
     __device__ void use_spill_staging(void* staging) {
@@ -228,6 +229,9 @@ public:
     // it, so the object can take another round of add().
     __device__ void flush() {
         if constexpr (S == Strategy::GlobalAtomics) return;
+        if constexpr (Spill) {
+            if (spill_ != nullptr && staged_ != 0) write_out_staged();
+        }
         __syncthreads();
         // e runs over the global layout (slot-major) so the atomics of a
         // wavefront touch consecutive addresses.
@@ -278,38 +282,51 @@ private:
     }
 
     // deposit() for a whole wavefront (lanes with slot < 0 have nothing): hits go to the table,
-    // misses are compacted into the wavefront's staging rows (slot, g[0..Width)) and written out
-    // with lane l on element l % Width of staged row l / Width, then the next 64 elements, ...
+    // misses are compacted into the wavefront's staging rows.
     __device__ __forceinline__ void deposit_together(int slot, const T (&g)[Width]) {
         const int row = slot >= 0 ? find_row(slot) : -1;
         if (row >= 0) {
 #pragma unroll
             for (int k = 0; k < Width; ++k) detail::atomic_add(table_ + k * capacity_ + row, static_cast<TableT>(g[k]));
         }
+        // Misses wait in the staging rows until these are full (or until flush()): a round of stores for
+        // the one or two misses of a typical call would cost more than the misses themselves.
         bool miss = slot >= 0 && row < 0;
         for (std::uint64_t missing = wave::ballot(miss); missing != 0; missing = wave::ballot(miss)) {
-            // this round: the first kStageRows lanes that still have a contribution without a row
             const unsigned before = __builtin_amdgcn_mbcnt_hi(static_cast<unsigned>(missing >> 32),
                                                               __builtin_amdgcn_mbcnt_lo(static_cast<unsigned>(missing), 0u));
-            if (miss && before < static_cast<unsigned>(kStageRows)) {
-                std::uint32_t* mine = spill_ + before * (Width + 1);
+            const unsigned room = static_cast<unsigned>(kStageRows) - staged_;
+            if (miss && before < room) {
+                std::uint32_t* mine = spill_ + (staged_ + before) * (Width + 1);
                 mine[0] = static_cast<std::uint32_t>(slot);
 #pragma unroll
                 for (int k = 0; k < Width; ++k) mine[1 + k] = __builtin_bit_cast(std::uint32_t, g[k]);
                 miss = false;
             }
-            __builtin_amdgcn_wave_barrier();
-            const int waiting = __builtin_popcountll(missing);
-            const int elements = (waiting < kStageRows ? waiting : kStageRows) * Width;
-            for (int e = static_cast<int>(wave::lane_id()); e < elements; e += 64) {
-                const int entry = e / Width, k = e - entry * Width;
-                const std::uint32_t* staged = spill_ + entry * (Width + 1);
-                const T value = __builtin_bit_cast(T, staged[1 + k]);
-                if (value != T(0))
-                    detail::atomic_add(global_ + static_cast<std::size_t>(staged[0]) * row_stride_ + k, value);
+            const unsigned waiting = static_cast<unsigned>(__builtin_popcountll(missing));
+            if (waiting <= room) {  // the same for every lane
+                staged_ += waiting;
+                break;
             }
-            __builtin_amdgcn_wave_barrier();
+            staged_ = static_cast<unsigned>(kStageRows);
+            write_out_staged();
         }
+    }
+
+    // The wavefront's staged rows (slot, g[0..Width)) go out with lane l on element l % Width of staged
+    // row l / Width, then the next 64 elements, ...
+    __device__ __forceinline__ void write_out_staged() {
+        __builtin_amdgcn_wave_barrier();
+        const int elements = static_cast<int>(staged_) * Width;
+        for (int e = static_cast<int>(wave::lane_id()); e < elements; e += 64) {
+            const int entry = e / Width, k = e - entry * Width;
+            const std::uint32_t* staged = spill_ + entry * (Width + 1);
+            const T value = __builtin_bit_cast(T, staged[1 + k]);
+            if (value != T(0))
+                detail::atomic_add(global_ + static_cast<std::size_t>(staged[0]) * row_stride_ + k, value);
+        }
+        __builtin_amdgcn_wave_barrier();
+        staged_ = 0;
     }
 
     // Level 1.  Take the slot of the first lane that is still waiting and find
@@ -353,6 +370,7 @@ private:
     int copies_base_;  // first row of the second copy
     int my_copy_;      // offset of this lane's copy of a hot row (0 for the first copy)
     std::uint32_t* spill_ = nullptr;
+    unsigned staged_ = 0;  // rows waiting in spill_; the same in every lane of a wavefront
 };
 
 // A leaf that reads its values like a VariableRef and sends its gradients to a
