@@ -22,7 +22,7 @@ if ROOT not in sys.path:
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published
 # HBM bytes per evaluation of the chain kernel, from FETCH_SIZE / WRITE_SIZE counter
 # passes scaled by a copy of known size (profiles/chain_single_kernel_hbm_traffic.md)
-MEASURED_TRAFFIC_BYTES_PER_EVAL = 52.001
+MEASURED_TRAFFIC_BYTES_PER_EVAL = 52.000
 TRAFFIC_SOURCE = {"profile": "profiles/chain_single_kernel_hbm_traffic.md", "bytes_per_eval": MEASURED_TRAFFIC_BYTES_PER_EVAL,
                   "note": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of `bench.py --counter-probe chain`, each scaled by a copy of "
                           "known size; a constant from that profile, not a reading of this run"}
@@ -119,16 +119,22 @@ def accumulate_report(ins, seed, with_oracle):
 
             ref = _oracle.load().accumulate_chain(host, slot.cpu().numpy(), num_slots, chain_in_double=True)
         for name, reps in (("auto", 10), ("wave_lds", 5), ("lds_f32", 5), ("global_atomics", 1)):
-            times = []
-            for _ in range(reps + (1 if reps > 1 else 0)):
-                grads.zero_()
-                a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                a.record()
+            # `reps` launches back to back between one pair of events (the sums simply keep growing), after a
+            # warm-up launch; then one launch from zero, which is the one checked below
+            grads.zero_()
+            if reps > 1:
                 accumulate.accumulate_chain_gradients(sub, slot, grads, name)
-                b.record()
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            for _ in range(reps):
+                accumulate.accumulate_chain_gradients(sub, slot, grads, name)
+            b.record()
+            torch.cuda.synchronize()
+            ms = a.elapsed_time(b) / reps
+            if reps > 1:
+                grads.zero_()
+                accumulate.accumulate_chain_gradients(sub, slot, grads, name)
                 torch.cuda.synchronize()
-                times.append(a.elapsed_time(b))
-            ms = sorted(times[1:] if reps > 1 else times)[len(times[1:] if reps > 1 else times) // 2]
             item = {"ms": ms, "GBps": (accumulate.BYTES_PER_THREAD * n + 24.0 * num_slots) / ms / 1e6}
             if ref is not None:
                 got = grads.cpu().numpy().astype(np.float64)
