@@ -301,7 +301,11 @@ int xad_trainer_create(const xad_training_config* config, int width, int height,
                        const float* target_rgb, xad_trainer** out);
 void xad_trainer_destroy(xad_trainer* trainer);
 /* Runs `iterations` iterations.  loss_out (host, may be NULL) receives the sum
- * of squared errors of the last iteration's rendering, taken before its update. */
+ * of squared errors of the last iteration's rendering, taken before its update.
+ * Only an iteration that reports its loss waits for the device.  Returns
+ * XAD_ERR_INCOMPLETE, with every iteration run and loss_out set, if the tile lists
+ * outgrew their buffers in an iteration since the last reported loss (that
+ * iteration's gradients lacked contributions; the buffers have been enlarged). */
 int xad_trainer_run(xad_trainer* trainer, int iterations, double* loss_out);
 /* Iterations completed so far (continues from the checkpoint after a load). */
 int xad_trainer_iteration(const xad_trainer* trainer);

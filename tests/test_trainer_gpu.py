@@ -89,6 +89,32 @@ def test_training_fits_the_test_pattern(gpu):
     t.close()
 
 
+def test_lists_that_outgrow_their_buffers_during_a_run_are_reported_and_the_run_goes_on(gpu):
+    """Iterations that do not report a loss never wait for the device, so a run whose Gaussians have grown
+    outgrows the tile lists' buffers unnoticed.  The run must finish, say so once its last iteration reads the
+    device's report, and work normally afterwards with the enlarged buffers."""
+    W = H = 256
+    target = trainer.test_pattern(W, H)
+    t = trainer.Trainer(_config(num_gaussians=4000), target)
+    t.run(2)  # sizes the buffers for the initial Gaussians (a few pixels across)
+    params = t.state()["params"]
+    params[2:4] += 2.0  # seven times as wide: about twenty times the pairs
+    t.set_params(params)
+    with pytest.warns(RuntimeWarning, match="outgrown their buffers"):
+        loss = t.run(8)
+    assert t.iteration == 10 and np.isfinite(loss)
+    state = t.state()
+    assert all(np.isfinite(v).all() for v in state.values() if isinstance(v, np.ndarray))
+    # the report has been taken and the buffers fit again: a rendering with every contribution
+    import warnings
+
+    with warnings.catch_warnings():
+        warnings.simplefilter("error")
+        again = t.run(1)
+    assert np.isfinite(again) and np.mean((t.image() - target) ** 2) * 3 * W * H == pytest.approx(again, rel=1e-3)
+    t.close()
+
+
 def test_checkpoint_round_trip_and_resume(gpu, tmp_path, xad):
     W, H, G = 80, 56, 400
     target = trainer.test_pattern(W, H)

@@ -10,6 +10,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libxad_hip.so")
 
 XAD_OK = 0
+XAD_ERR_INCOMPLETE = 5
 
 
 class XadError(RuntimeError):

@@ -188,7 +188,7 @@ std::uint32_t grown(std::uint32_t pairs) {
 //     enlarged and the binning is redone).
 // Otherwise nothing is read back: an overflow or a depth that changed against the caller's promise is
 // left in the sticky status words for the next call that waits anyway.
-int bin(xad_splat_context* c, const float* params, const float* depth, hipStream_t s) {
+int bin(xad_splat_context* c, const float* params, const float* depth, hipStream_t s, bool first_attempt = true) {
     int current = -1;
     XAD_HIP_TRY(hipGetDevice(&current));
     XAD_REQUIRE(current == c->device, "splat: the context belongs to device %d, but device %d is current", c->device, current);
@@ -198,11 +198,11 @@ int bin(xad_splat_context* c, const float* params, const float* depth, hipStream
     const bool had_order = c->order_valid && c->depth_mode != XAD_SPLAT_DEPTH_EVERY_STEP;
     if (!had_order)
         if (int st = order_by_depth(c, depth, s)) return st;
-    auto project = [&]() {
+    auto project = [&](bool first_of_step) {
         return launch_project(s, c->G, params, depth, c->ordered_depth, c->rank, c->status, c->width, c->height, c->records,
-                              c->rects, c->rects_by_depth, c->record_grads, c->loss);
+                              c->rects, c->rects_by_depth, c->record_grads, c->loss, first_of_step);
     };
-    if (int st = project()) return st;
+    if (int st = project(first_attempt)) return st;
     mark(c, 1, s);
     const bool check_depth = c->depth_mode == XAD_SPLAT_DEPTH_CHECKED && had_order;
     if (check_depth) {
@@ -218,7 +218,7 @@ int bin(xad_splat_context* c, const float* params, const float* depth, hipStream
         XAD_HIP_TRY(hipEventSynchronize(c->report_ready));
         if (c->report->status[kStatusDepthChanged] != 0) {
             if (int st = order_by_depth(c, depth, s)) return st;
-            if (int st = project()) return st;  // the rectangles in the new order
+            if (int st = project(false)) return st;  // the rectangles in the new order
             if (int st = bin_lists(c, s, true)) return st;
         }
     }
@@ -371,8 +371,9 @@ extern "C" int xad_splat_step(xad_splat_context* c, const float* params, const f
     const char* who = "xad_splat_step";
     XAD_REQUIRE(c && params && depth && target && image && grads, "%s: null argument", who);
     hipStream_t s = xad::as_stream(stream);
+    bool earlier_steps_overflowed = false;
     for (int attempt = 0;; ++attempt) {
-        if (int st = bin(c, params, depth, s)) return st;
+        if (int st = bin(c, params, depth, s, attempt == 0)) return st;
         if (int st = launch_render_forward(s, c->width, c->height, c->range_begin, c->range_end, c->list, c->records, image,
                                            c->final_T, c->n_contrib, c->segments, c->segment_state))
             return st;
@@ -388,7 +389,9 @@ extern "C" int xad_splat_step(xad_splat_context* c, const float* params, const f
         // the loss is read back, and with it what the device has to report
         if (int st = fetch_report(c, s)) return st;
         if (c->report->status[kStatusOverflow] != 0 && attempt == 0) {
-            // this very step did not fit (the scene grew): enlarge the lists and do it again
+            // this very step did not fit (the scene grew): enlarge the lists and do it again.  Whether steps
+            // before it overflowed too is in the word the step saved when it began.
+            earlier_steps_overflowed = c->report->status[kStatusStickyBefore] != 0;
             if (int st = size_pair_buffers(c, grown(c->pairs > c->plan.capacity ? c->pairs : c->plan.capacity * 2))) return st;
             if (int st = clear_status(c, s, kStatusOverflowSticky, 1)) return st;
             c->report->status[kStatusOverflowSticky] = 0;
@@ -402,6 +405,11 @@ extern "C" int xad_splat_step(xad_splat_context* c, const float* params, const f
         break;
     }
     collect_times(c, 5);
+    if (earlier_steps_overflowed)
+        return xad::fail(XAD_ERR_INCOMPLETE,
+                         "%s: a call that did not wait for the device produced more pairs than the lists held; its image and "
+                         "gradients were incomplete.  The lists have been enlarged (this step is complete)",
+                         who);
     return XAD_OK;
 }
 

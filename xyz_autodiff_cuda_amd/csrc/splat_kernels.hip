@@ -35,8 +35,11 @@ __global__ void __launch_bounds__(256) project_kernel(int G, const float* __rest
                                                       std::uint32_t* __restrict__ status, int width, int height,
                                                       Record* __restrict__ records, TileRect* __restrict__ rects,
                                                       TileRect* __restrict__ rects_by_depth,
-                                                      float* __restrict__ record_grads, double* __restrict__ loss) {
+                                                      float* __restrict__ record_grads, double* __restrict__ loss,
+                                                      bool first_of_step) {
     const int g = blockIdx.x * 256 + threadIdx.x;
+    // what the steps before this one left in the sticky overflow word (this step's own binning may add to it)
+    if (first_of_step && g == 0) status[kStatusStickyBefore] = status[kStatusOverflowSticky];
     // what the compositing backward adds into starts from zero: the parts of the loss, this Gaussian's accumulator row
     if (blockIdx.x == 0 && threadIdx.x < kLossParts) loss[kLossStride * (1 + threadIdx.x)] = 0.0;
     if (g >= G) return;
@@ -695,9 +698,9 @@ __global__ void __launch_bounds__(256) gaussian_backward_kernel(int G, const flo
 
 int launch_project(hipStream_t s, int G, const float* params, const float* depth, const float* ordered_depth,
                    const std::uint32_t* rank, std::uint32_t* status, int width, int height, Record* records, TileRect* rects,
-                   TileRect* rects_by_depth, float* record_grads, double* loss) {
+                   TileRect* rects_by_depth, float* record_grads, double* loss, bool first_of_step) {
     hipLaunchKernelGGL(project_kernel, dim3(xad::blocks_for(G, 256)), dim3(256), 0, s, G, params, depth, ordered_depth, rank,
-                       status, width, height, records, rects, rects_by_depth, record_grads, loss);
+                       status, width, height, records, rects, rects_by_depth, record_grads, loss, first_of_step);
     XAD_HIP_TRY(hipGetLastError());
     return XAD_OK;
 }

@@ -17,7 +17,8 @@ enum : int {
     kStatusSuperPairs = 2,    // (supertile, Gaussian) pairs
     kStatusDepthChanged = 3,  // 1 if a depth differed from the depths the kept order was computed from
     kStatusOverflowSticky = 4,  // largest pair count of any step that overflowed since the host last cleared this word
-    kStatusWords = 5,
+    kStatusStickyBefore = 5,    // that word as it stood when the last step began: what steps before it left there
+    kStatusWords = 6,
 };
 
 // Also sets status[kStatusDepthChanged] if any depth differs (bitwise) from ordered_depth, and zeroes
@@ -25,7 +26,7 @@ enum : int {
 // rank[g] = position of Gaussian g in the depth order: the rectangle is also written to rects_by_depth[rank[g]].
 int launch_project(hipStream_t s, int G, const float* params, const float* depth, const float* ordered_depth,
                    const std::uint32_t* rank, std::uint32_t* status, int width, int height, Record* records, TileRect* rects,
-                   TileRect* rects_by_depth, float* record_grads, double* loss);
+                   TileRect* rects_by_depth, float* record_grads, double* loss, bool first_of_step);
 // Depth order: keys[g] = order-preserving bits of depth[g], identity[g] = g; the stable sort of
 // those pairs gives by_depth; rank is its inverse (rank[by_depth[i]] = i).
 int launch_depth_keys(hipStream_t s, int G, const float* depth, std::uint32_t* keys, std::uint32_t* identity);

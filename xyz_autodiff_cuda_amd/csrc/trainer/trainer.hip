@@ -147,16 +147,28 @@ extern "C" int xad_trainer_run(xad_trainer* t, int iterations, double* loss_out)
     const xad_training_config& c = t->config;
     const float learning_rates[9] = {c.lr_center, c.lr_center, c.lr_scale, c.lr_scale, c.lr_rotation,
                                      c.lr_color,  c.lr_color,  c.lr_color, c.lr_opacity};
+    int late = XAD_OK;
     for (int i = 0; i < iterations; ++i) {
         double* loss = (i + 1 == iterations) ? loss_out : nullptr;
-        if (int st = xad_splat_step(t->splat, t->params(), t->depth(), t->target, t->image, t->grads(), loss, t->stream))
-            return st;
+        int st = xad_splat_step(t->splat, t->params(), t->depth(), t->target, t->image, t->grads(), loss, t->stream);
+        if (st == XAD_ERR_INCOMPLETE) {
+            // this step is complete (a step that asks for its loss always is); the report is about earlier
+            // iterations, whose updates have been applied: the run goes on and the caller is told at the end
+            late = st;
+            st = XAD_OK;
+        }
+        if (st) return st;
         if (int st = xad_adam_step_f32(t->g(), 9, t->params(), t->grads(), t->m(), t->v(), learning_rates, c.beta1,
                                        c.beta2, c.epsilon, t->iteration + 1, t->stream))
             return st;
         ++t->iteration;
     }
     XAD_HIP_TRY(hipStreamSynchronize(t->stream));
+    if (late)
+        return xad::fail(late,
+                         "xad_trainer_run: all %d iterations were run, but in some iteration since the last reported loss the "
+                         "tile lists had outgrown their buffers and its gradients lacked contributions; the buffers have been enlarged",
+                         iterations);
     return XAD_OK;
 }
 

@@ -6,6 +6,7 @@ training_config.cpp, image_utils.cpp} in xyz-autodiff-cuda.  The command-line
 program built next to the library, xad_splat_train, uses the same entry points.
 """
 import ctypes
+import warnings
 import os
 
 import numpy as np
@@ -117,7 +118,12 @@ class Trainer:
 
     def run(self, iterations, want_loss=True):
         loss = ctypes.c_double(0.0)
-        _lib.check(self._lib.xad_trainer_run(self._handle, int(iterations), ctypes.byref(loss) if want_loss else None), "xad_trainer_run")
+        status = self._lib.xad_trainer_run(self._handle, int(iterations), ctypes.byref(loss) if want_loss else None)
+        if status == _lib.XAD_ERR_INCOMPLETE:
+            # every iteration has run; some earlier one lacked contributions (buffers outgrown, since enlarged)
+            warnings.warn(self._lib.xad_last_error().decode("utf-8", "replace"), RuntimeWarning)
+        else:
+            _lib.check(status, "xad_trainer_run")
         return loss.value if want_loss else None
 
     @property
