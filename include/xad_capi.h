@@ -177,6 +177,14 @@ int xad_accumulate_chain_gradients_f32(int strategy, size_t n,
  * and gradients lack the pairs that did not fit; the lists are enlarged at that
  * point), XAD_ERR_INVALID_ARGUMENT if a depth changed under the static promise.
  * The outputs of the call that returns such a status are themselves complete.
+ *
+ * Recording.  In XAD_SPLAT_DEPTH_STATIC mode, after a step with loss_out has
+ * returned (the lists are sized then), xad_splat_step with loss_out == NULL is a
+ * fixed sequence of kernel launches on `stream`, with no allocation, copy or fill
+ * and no host-side state that a launch depends on: it may be recorded by HIP
+ * stream capture and the graph replayed, for as long as the context is used by
+ * nothing else in between that changes its buffers (a call that reports
+ * XAD_ERR_INCOMPLETE enlarges them: record again after it).  Profiling must be off.
  */
 typedef struct xad_splat_context xad_splat_context;
 int xad_splat_create(int width, int height, int num_gaussians, size_t pair_capacity_hint,

@@ -363,6 +363,63 @@ def test_steps_that_do_not_wait(gpu, oracle, mode):
     ctx.close()
 
 
+@pytest.mark.parametrize("G,W,H,scale", [
+    (3000, 256, 192, (1.0, 20.0)),    # few tiles: the backward walk in pieces
+    (20000, 1100, 1100, (1.0, 24.0)),  # many tiles: one wavefront per tile
+])
+def test_a_recorded_step_can_be_replayed(gpu, oracle, G, W, H, scale):
+    """A step that asks for no loss, in a context whose buffers are sized and whose depths are promised constant, is
+    kernel launches only and keeps no host-side state that a launch depends on: recorded into a HIP graph, it can be
+    replayed.  Every replay, with the parameters changed in between by ordinary launches, against the same step
+    launched the ordinary way."""
+    import torch
+
+    from xyz_autodiff_cuda_amd import splat
+
+    params, depth = random_scene(G, W, H, seed=17, scale_px=scale)
+    target = np.random.default_rng(6).uniform(0, 1, (H, W, 3)).astype(np.float32)
+    p, d, t = (torch.from_numpy(a).to(gpu) for a in (params, depth, target))
+    image, grads = torch.empty(H, W, 3, device=gpu), torch.empty(9, G, device=gpu)
+    m, v = torch.zeros_like(p), torch.zeros_like(p)
+    ctx = splat.SplatContext(W, H, G, depth_mode="static")
+    eager = splat.SplatContext(W, H, G)
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        ctx.step(p, d, t, image, grads)  # sizes the buffers
+        ctx.step(p, d, t, image, grads, want_loss=False)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=stream):
+        ctx.step(p, d, t, image, grads, want_loss=False)
+    torch.cuda.synchronize()
+    for replay in range(4):
+        if replay:
+            splat.adam_step(p, grads, m, v, 2e-2, replay)  # other parameters for the next replay
+            torch.cuda.synchronize()
+        image.fill_(-1.0)
+        grads.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        # the same step launched the ordinary way, in a context of its own: the same image bit for bit, the same
+        # gradients up to the order of the atomic sums
+        want_image, want_grads, want_loss = eager.step(p, d, t)
+        torch.cuda.synchronize()
+        assert torch.equal(image, want_image), replay
+        scale_g = want_grads.abs().amax(dim=0) + 1e-20
+        # (sums of terms of either sign, added in another order: 1e-4 of their mass, which in a dense scene
+        # is several times the sum itself)
+        off = (grads - want_grads).abs() / scale_g
+        assert float(off.max()) < 1e-2 and float((off < 1e-4).float().mean()) > 0.999, (replay, float(off.max()))
+        assert ctx.stats()["pairs"] == eager.stats()["pairs"], replay
+    # the last replay against the oracle, and the context outside the graph
+    ref = oracle.splat_step(W, H, p.cpu().numpy(), depth, target, np.float32)
+    assert np.abs(image.cpu().numpy() - ref["image"]).max() < 2e-5 and ctx.stats()["pairs"] == ref["pairs"]
+    _, _, loss = ctx.step(p, d, t, image, grads)
+    assert abs(loss - ref["loss"]) <= 1e-5 * ref["loss"] and abs(loss - want_loss) <= 1e-6 * want_loss
+    ctx.close()
+    eager.close()
+
+
 def test_static_mode_reports_a_changed_depth(gpu, xad):
     import torch
 

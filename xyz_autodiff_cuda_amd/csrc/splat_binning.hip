@@ -50,6 +50,10 @@ __device__ __forceinline__ std::uint32_t read_lane(std::uint32_t v, int lane) {
 // Blocks take tickets, so a block only ever waits for blocks that are already running.  The state
 // words carry the launch's epoch, so nothing has to be cleared between launches: a word of another
 // epoch simply is not there yet.  data[n] receives the total.
+// Tickets and epoch live in three control words on the device (tickets given out, blocks finished, epoch);
+// the block that finishes last puts the first two back to zero and moves the epoch on.  Nothing about
+// a launch depends on what the host knows of earlier launches, so a recorded launch can be replayed.
+enum : int { kScanTickets = 0, kScanFinished = 1, kScanEpoch = 2 };
 constexpr unsigned kScanBlock = 1024;
 constexpr unsigned kScanItems = 16;
 constexpr unsigned kScanTile = kScanBlock * kScanItems;  // few, large blocks: the chain of look-backs stays short
@@ -59,14 +63,17 @@ __device__ __forceinline__ std::uint64_t scan_word(std::uint32_t epoch, std::uin
 }
 
 __global__ void __launch_bounds__(kScanBlock) scan_kernel(std::uint32_t* __restrict__ data, std::uint32_t n,
-                                                          std::uint64_t* __restrict__ state, std::uint32_t* __restrict__ tickets,
-                                                          std::uint32_t ticket_base, std::uint32_t epoch) {
+                                                          std::uint64_t* __restrict__ state, std::uint32_t* __restrict__ control) {
     __shared__ std::uint32_t wave_total[kScanBlock / 64];
-    __shared__ std::uint32_t block_index, block_exclusive;
+    __shared__ std::uint32_t block_index, block_exclusive, launch_epoch;
     const unsigned t = threadIdx.x;
-    if (t == 0) block_index = atomicAdd(tickets, 1u) - ticket_base;
+    if (t == 0) {
+        launch_epoch = __hip_atomic_load(control + kScanEpoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // before the ticket: it moves on only after every block has one
+        block_index = atomicAdd(control + kScanTickets, 1u);
+    }
     __syncthreads();
     const std::uint32_t b = block_index;
+    const std::uint32_t epoch = launch_epoch;
     const std::uint32_t first = b * kScanTile + t * kScanItems;
 
     std::uint32_t v[kScanItems];
@@ -150,6 +157,14 @@ __global__ void __launch_bounds__(kScanBlock) scan_kernel(std::uint32_t* __restr
             if (first + k < n) data[first + k] = running;
             running += v[k];
         }
+    }
+    // the block that finishes last leaves the control words ready for the next launch (epoch 0 is never
+    // used: the state words start out as zero)
+    if (t == 0 && atomicAdd(control + kScanFinished, 1u) == gridDim.x - 1) {
+        const std::uint32_t next = (epoch + 1) & 0x3fffffffu;
+        control[kScanTickets] = 0;
+        control[kScanFinished] = 0;
+        control[kScanEpoch] = next == 0 ? 1u : next;
     }
 }
 
@@ -480,15 +495,12 @@ std::size_t bin_scan_state_words(const BinPlan& p) {
 
 namespace {
 
-int launch_scan(hipStream_t s, std::uint32_t* data, std::size_t n, BinScratch& scratch) {
+int launch_scan(hipStream_t s, std::uint32_t* data, std::size_t n, const BinScratch& scratch) {
     XAD_REQUIRE(n > 0 && n < (std::size_t(1) << 32) - 2 * kScanTile, "splat binning: %zu counts do not fit the 32-bit scan", n);
     const unsigned blocks = static_cast<unsigned>((n + kScanTile - 1) / kScanTile);
-    scratch.epoch = (scratch.epoch + 1) & 0x3fffffffu;
-    if (scratch.epoch == 0) scratch.epoch = 1;  // state words start as zero: epoch 0 is never used
     hipLaunchKernelGGL(scan_kernel, dim3(blocks), dim3(kScanBlock), 0, s, data, static_cast<std::uint32_t>(n), scratch.scan_state,
-                       scratch.tickets, scratch.tickets_taken, scratch.epoch);
+                       scratch.scan_control);
     XAD_HIP_TRY(hipGetLastError());
-    scratch.tickets_taken += blocks;  // wraps like the device counter
     return XAD_OK;
 }
 

@@ -99,7 +99,7 @@ void carve_fixed(xad_splat_context* c, char* base, std::size_t* bytes) {
     c->record_grads = k.take<float>(G * kRecordGradStride);
     c->loss = k.take<double>(kLossWords);
     c->status = k.take<std::uint32_t>(kStatusWords);
-    c->bin.tickets = k.take<std::uint32_t>(1);
+    c->bin.scan_control = k.take<std::uint32_t>(kScanControlWords);
     c->depth_sort_temp = k.take<char>(c->depth_sort_bytes ? c->depth_sort_bytes : 16);
     *bytes = k.used;
 }
@@ -135,6 +135,7 @@ int size_pair_buffers(xad_splat_context* c, std::uint32_t capacity) {
     carve_paired(c, static_cast<char*>(base), &bytes);
     // the scan's state words must not look like words of a coming epoch
     XAD_HIP_TRY(hipMemset(c->bin.scan_state, 0, bin_scan_state_words(c->plan) * sizeof(std::uint64_t)));
+    XAD_HIP_TRY(hipDeviceSynchronize());  // the fill is not on the caller's stream
     return XAD_OK;
 }
 
@@ -304,8 +305,11 @@ extern "C" int xad_splat_create(int width, int height, int num_gaussians, std::s
     if (hipMalloc(&c->fixed, bytes) != hipSuccess) st = xad::fail(XAD_ERR_HIP, "%s: hipMalloc of %zu bytes failed", who, bytes);
     if (st == XAD_OK) {
         carve_fixed(c, static_cast<char*>(c->fixed), &bytes);
-        // status words, the scan's ticket counter and the tile ranges start from zero
+        // status words, the scan's control words and the tile ranges start from zero; the scan's epoch from one
         if (hipMemset(c->fixed, 0, bytes) != hipSuccess) st = xad::fail(XAD_ERR_HIP, "%s: hipMemset failed", who);
+        const std::uint32_t control[kScanControlWords] = {0u, 0u, 1u};
+        if (st == XAD_OK && hipMemcpy(c->bin.scan_control, control, sizeof(control), hipMemcpyHostToDevice) != hipSuccess)
+            st = xad::fail(XAD_ERR_HIP, "%s: hipMemcpy failed", who);
     }
     if (st == XAD_OK && hipHostMalloc(reinterpret_cast<void**>(&c->report), sizeof(HostReport)) != hipSuccess)
         st = xad::fail(XAD_ERR_HIP, "%s: pinned allocation failed", who);

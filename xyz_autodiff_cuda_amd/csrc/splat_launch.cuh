@@ -44,15 +44,14 @@ struct BinPlan {
     std::uint32_t capacity_a;      // (supertile, Gaussian) pairs level A may produce: at most capacity (the buffer's size)
     std::uint32_t waves_b;         // wavefronts launched at level B: capacity_a / kBinRangeB + supers
 };
+constexpr int kScanControlWords = 3;
 struct BinScratch {
     std::uint32_t* matrix_a = nullptr;    // bin_matrix_a_words: counts, then offsets, per (supertile, range)
     std::uint32_t* matrix_b = nullptr;    // bin_matrix_b_words: the same per (tile, range of its supertile's list)
     std::uint32_t* list_a = nullptr;      // capacity: the supertiles' lists
     std::uint32_t* first_wave = nullptr;  // supers + 1
     std::uint64_t* scan_state = nullptr;  // bin_scan_state_words, zero before the first launch
-    std::uint32_t* tickets = nullptr;     // one word, zero before the first launch
-    std::uint32_t tickets_taken = 0;      // host mirror of *tickets
-    std::uint32_t epoch = 0;              // of the last scan launched
+    std::uint32_t* scan_control = nullptr;  // kScanControlWords: tickets given out, blocks finished (both zero between launches), epoch (never zero)
 };
 // The buffers are sized by a plan with capacity_a = capacity; a plan with a smaller capacity_a (once the host
 // has seen how many supertile pairs a scene produces) uses less of them and launches fewer wavefronts.
