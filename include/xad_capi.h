@@ -99,7 +99,12 @@ int xad_host_chain_forward_backward_f64(size_t n,
  *   GLOBAL_ATOMICS  one global atomic per thread per element: the pattern of
  *                   VariableRef::add_grad (include/xyz_autodiff/variable.cuh:48-50;
  *                   tests/test_parallel_gradient_accumulation.cu:25-49);
- *   AUTO            LDS (the measured optimum at every slot count from 1 to 262 144);
+ *   AUTO            the fastest measured at every slot count from 1 to 1 Mi: LDS while
+ *                   one fp64 table holds every slot (3072 slots); beyond that the
+ *                   whole LDS of a CU as fp64 rows for the first ~3000 slots (the
+ *                   hottest 32 in several copies), every other slot's contributions
+ *                   gathered per wavefront in LDS and written to HBM sixteen rows
+ *                   at a time, coalesced.  Every input is read once;
  *   LDS             per-block table of partial sums in LDS, written out once per
  *                   block (the reference's shared-memory pattern,
  *                   tests/test_shared_memory_atomic.cu:29-64, made persistent).
