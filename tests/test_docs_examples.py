@@ -1,4 +1,4 @@
-"""The device-code example of INTEGRATION.md is compiled as it stands in the document."""
+"""The device-code example of the integration guide is compiled as it stands in the document."""
 import os
 import re
 import shutil
@@ -15,7 +15,7 @@ def test_integration_example_compiles_for_gfx950(tmp_path):
         pytest.skip("hipcc is not installed")
     text = open(os.path.join(ROOT, "INTEGRATION.md")).read()
     block = re.search(r"```cpp\n(#include <xyz_autodiff/xyz_autodiff\.cuh>.*?)```", text, re.S)
-    assert block, "the example kernel is missing from INTEGRATION.md"
+    assert block, "the example kernel is missing from the integration guide"
     src = tmp_path / "example.hip"
     src.write_text(block.group(1))
     cmd = [hipcc, "--offload-arch=gfx950", "-std=c++20", "-O1", "-I" + os.path.join(ROOT, "include"), "-munsafe-fp-atomics",
@@ -26,14 +26,14 @@ def test_integration_example_compiles_for_gfx950(tmp_path):
 
 
 def test_integration_host_stub_compiles(tmp_path):
-    """The C++ stubs of INTEGRATION.md against include/xad_capi.h (syntax and types only)."""
+    """The C++ stubs of the integration guide against include/xad_capi.h (syntax and types only)."""
     gxx = shutil.which("g++")
     hip_include = "/opt/rocm/include"
     if not gxx or not os.path.exists(os.path.join(hip_include, "hip", "hip_runtime_api.h")):
         pytest.skip("g++ or the HIP headers are not installed")
     text = open(os.path.join(ROOT, "INTEGRATION.md")).read()
     block = re.search(r"```cpp\n(// replaces launch_gaussian_splatting.*?)```", text, re.S)
-    assert block, "the host stub is missing from INTEGRATION.md"
+    assert block, "the host stub is missing from the integration guide"
     prelude = ("#include <cstddef>\n#include <stdexcept>\n#include <hip/hip_runtime_api.h>\n"
                "static float lr_pos = 1e-2f, lr_scale = 1e-2f, lr_rot = 1e-2f, lr_col = 1e-2f, lr_opacity = 1e-2f;\n")
     src = tmp_path / "stub.cpp"

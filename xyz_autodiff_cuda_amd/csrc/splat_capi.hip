@@ -43,6 +43,7 @@ struct xad_splat_context {
     std::uint32_t *range_begin = nullptr, *range_end = nullptr;         // tiles each, adjacent
     float* final_T = nullptr;
     std::uint32_t* n_contrib = nullptr;
+    std::uint32_t* tile_order = nullptr;  // 8 * ceil(tiles / 8): which tile each block of the compositing kernels takes
     int segments = 1;                 // pieces a tile's list is cut into for the backward walk
     float4* segment_state = nullptr;  // segments x pixels when segments > 1
     float* record_grads = nullptr;  // G x kRecordGradStride
@@ -95,6 +96,7 @@ void carve_fixed(xad_splat_context* c, char* base, std::size_t* bytes) {
     c->range_end = c->range_begin ? c->range_begin + c->tiles : nullptr;
     c->final_T = k.take<float>(pixels);
     c->n_contrib = k.take<std::uint32_t>(pixels);
+    c->tile_order = k.take<std::uint32_t>(static_cast<std::size_t>((c->tiles + 7) / 8) * 8);
     c->segment_state = c->segments > 1 ? k.take<float4>(pixels * static_cast<std::size_t>(c->segments)) : nullptr;
     c->record_grads = k.take<float>(G * kRecordGradStride);
     c->loss = k.take<double>(kLossWords);
@@ -363,7 +365,7 @@ extern "C" int xad_splat_forward(xad_splat_context* c, const float* params, cons
     hipStream_t s = xad::as_stream(stream);
     if (int st = bin(c, params, depth, s)) return st;
     if (int st = launch_render_forward(s, c->width, c->height, c->range_begin, c->range_end, c->list, c->records, image,
-                                       c->final_T, c->n_contrib, c->segments, c->segment_state))
+                                       c->final_T, c->n_contrib, c->segments, c->segment_state, c->tile_order))
         return st;
     mark(c, 3, s);
     collect_times(c, 3);
@@ -379,12 +381,12 @@ extern "C" int xad_splat_step(xad_splat_context* c, const float* params, const f
     for (int attempt = 0;; ++attempt) {
         if (int st = bin(c, params, depth, s, attempt == 0)) return st;
         if (int st = launch_render_forward(s, c->width, c->height, c->range_begin, c->range_end, c->list, c->records, image,
-                                           c->final_T, c->n_contrib, c->segments, c->segment_state))
+                                           c->final_T, c->n_contrib, c->segments, c->segment_state, c->tile_order))
             return st;
         mark(c, 3, s);
         if (int st = launch_render_backward(s, c->width, c->height, c->range_begin, c->range_end, c->list, c->records, image,
                                             target, c->final_T, c->n_contrib, c->record_grads, c->loss, c->segments,
-                                            c->segment_state))
+                                            c->segment_state, c->tile_order))
             return st;
         mark(c, 4, s);
         if (int st = launch_gaussian_backward(s, c->G, params, c->record_grads, grads, c->loss)) return st;

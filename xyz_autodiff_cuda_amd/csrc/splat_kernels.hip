@@ -133,6 +133,63 @@ __device__ __forceinline__ int tile_of_block(int block, int tiles) {
     return t;  // may be >= tiles for the padding blocks of the last band
 }
 
+// Within its band every XCD takes its tiles longest list first: blocks are started in order of their
+// index, and a tile with a long list that starts late leaves the SIMDs around it idle at the end of the
+// launch.  One block per band: a histogram of the list lengths (in units of eight entries) in LDS, a
+// descending prefix, and a scatter; the order within a bucket is whatever the atomics make it.
+// order[band * per_band + i] = the tile that the band's i-th block takes, or ~0 for none.
+constexpr int kOrderBuckets = 512;
+__global__ void __launch_bounds__(1024) tile_order_kernel(int tiles, const std::uint32_t* __restrict__ range_begin,
+                                                          const std::uint32_t* __restrict__ range_end,
+                                                          std::uint32_t* __restrict__ order) {
+    __shared__ std::uint32_t bucket[kOrderBuckets];
+    const int per = (tiles + 7) / 8;
+    const int band_first = static_cast<int>(blockIdx.x) * per;
+    const int band_last = band_first + per < tiles ? band_first + per : (band_first < tiles ? tiles : band_first);  // an empty band for few tiles
+    const int t = static_cast<int>(threadIdx.x);
+    for (int k = t; k < kOrderBuckets; k += 1024) bucket[k] = 0;
+    __syncthreads();
+    auto bucket_of = [&](int tile) {
+        const std::uint32_t length = range_end[tile] - range_begin[tile];
+        const std::uint32_t b = length >> 3;
+        return kOrderBuckets - 1 - static_cast<int>(b < kOrderBuckets - 1 ? b : kOrderBuckets - 1);  // longest first
+    };
+    for (int tile = band_first + t; tile < band_last; tile += 1024) atomicAdd(&bucket[bucket_of(tile)], 1u);
+    __syncthreads();
+    // exclusive prefix over the buckets, by the first wavefront: eight buckets per lane
+    if (t < 64) {
+        std::uint32_t mine[kOrderBuckets / 64], sum = 0;
+#pragma unroll
+        for (int k = 0; k < kOrderBuckets / 64; ++k) {
+            mine[k] = bucket[t * (kOrderBuckets / 64) + k];
+            sum += mine[k];
+        }
+        std::uint32_t inclusive = sum;
+#pragma unroll
+        for (int step = 1; step < 64; step *= 2) {
+            const std::uint32_t other = __shfl_up(inclusive, step, 64);
+            if (t >= step) inclusive += other;
+        }
+        std::uint32_t running = inclusive - sum;
+#pragma unroll
+        for (int k = 0; k < kOrderBuckets / 64; ++k) {
+            bucket[t * (kOrderBuckets / 64) + k] = running;
+            running += mine[k];
+        }
+    }
+    __syncthreads();
+    for (int tile = band_first + t; tile < band_last; tile += 1024)
+        order[band_first + atomicAdd(&bucket[bucket_of(tile)], 1u)] = static_cast<std::uint32_t>(tile);
+    for (int k = band_last - band_first + t; k < per; k += 1024) order[band_first + k] = ~0u;  // the last band may be short
+}
+
+// Tile of a block: block b belongs to XCD b % 8 and is that XCD's (b / 8)-th block.
+__device__ __forceinline__ int ordered_tile_of_block(int block, int tiles, const std::uint32_t* __restrict__ order) {
+    const int per = (tiles + 7) / 8;
+    const std::uint32_t tile = order[(block % 8) * per + block / 8];
+    return tile == ~0u ? tiles : static_cast<int>(tile);
+}
+
 // ---------------------------------------------------------------------------
 // Compositing kernels.  One wavefront per tile; lane l owns the four
 // horizontally adjacent pixels x = 4 (l % 4) .. +3 of row y = l / 4.  Four
@@ -246,9 +303,10 @@ __global__ void __launch_bounds__(kChunk) render_forward_kernel(
     int width, int height, int tiles_x, int tiles, const std::uint32_t* __restrict__ range_begin,
     const std::uint32_t* __restrict__ range_end, const std::uint32_t* __restrict__ sorted_ids,
     const Record* __restrict__ records, float* __restrict__ image, float* __restrict__ final_T,
-    std::uint32_t* __restrict__ n_contrib, int segments, float4* __restrict__ segment_state) {
+    std::uint32_t* __restrict__ n_contrib, int segments, float4* __restrict__ segment_state,
+    const std::uint32_t* __restrict__ tile_order) {
     __shared__ Staged staged[kChunk];
-    const int tile = tile_of_block(blockIdx.x, tiles);
+    const int tile = ordered_tile_of_block(blockIdx.x, tiles, tile_order);
     if (tile >= tiles) return;
     const int lane = threadIdx.x;
     const int x0 = (tile % tiles_x) * kTile + (lane & 3) * kLanePixels;
@@ -456,7 +514,8 @@ __global__ void __launch_bounds__(kChunk) render_backward_kernel(
     const std::uint32_t* __restrict__ range_end, const std::uint32_t* __restrict__ sorted_ids,
     const Record* __restrict__ records, const float* __restrict__ image, const float* __restrict__ target,
     const float* __restrict__ final_T, const std::uint32_t* __restrict__ n_contrib, float* __restrict__ record_grads,
-    double* __restrict__ loss, int segments, const float4* __restrict__ segment_state) {
+    double* __restrict__ loss, int segments, const float4* __restrict__ segment_state,
+    const std::uint32_t* __restrict__ tile_order) {
     __shared__ Staged staged[kChunk];
     __shared__ std::uint32_t staged_id[kChunk];
     // Row sums wait here until a group of kPark list entries is complete.  Small on purpose: LDS per
@@ -468,7 +527,7 @@ __global__ void __launch_bounds__(kChunk) render_backward_kernel(
     // segment (the late segments are the ones that often have nothing to walk)
     const unsigned blocks_per_segment = kSplit ? gridDim.x / static_cast<unsigned>(segments) : gridDim.x;
     const int segment = kSplit ? static_cast<int>(blockIdx.x / blocks_per_segment) : 0;
-    const int tile = tile_of_block(static_cast<int>(blockIdx.x % blocks_per_segment), tiles);
+    const int tile = ordered_tile_of_block(static_cast<int>(blockIdx.x % blocks_per_segment), tiles, tile_order);
     if (tile >= tiles) return;
     const int lane = threadIdx.x;
     const int x0 = (tile % tiles_x) * kTile + (lane & 3) * kLanePixels;
@@ -726,16 +785,20 @@ int render_segments(int width, int height) {
 
 int launch_render_forward(hipStream_t s, int width, int height, const std::uint32_t* range_begin,
                           const std::uint32_t* range_end, const std::uint32_t* sorted_ids, const Record* records,
-                          float* image, float* final_T, std::uint32_t* n_contrib, int segments, float4* segment_state) {
+                          float* image, float* final_T, std::uint32_t* n_contrib, int segments, float4* segment_state,
+                          std::uint32_t* tile_order) {
     const int tiles_x = (width + kTile - 1) / kTile, tiles = tiles_x * ((height + kTile - 1) / kTile);
+    // the order both compositing kernels of this step take the tiles in
+    hipLaunchKernelGGL(tile_order_kernel, dim3(8), dim3(1024), 0, s, tiles, range_begin, range_end, tile_order);
+    XAD_HIP_TRY(hipGetLastError());
     XAD_REQUIRE(segments >= 1 && (segments == 1 || segment_state), "splat: a split walk needs its per-segment state");
     if (segments > 1)
         hipLaunchKernelGGL(render_forward_kernel<true>, dim3(padded_tile_blocks(tiles)), dim3(kChunk), 0, s, width, height,
                            tiles_x, tiles, range_begin, range_end, sorted_ids, records, image, final_T, n_contrib, segments,
-                           segment_state);
+                           segment_state, tile_order);
     else
         hipLaunchKernelGGL(render_forward_kernel<false>, dim3(padded_tile_blocks(tiles)), dim3(kChunk), 0, s, width, height,
-                           tiles_x, tiles, range_begin, range_end, sorted_ids, records, image, final_T, n_contrib, 1, nullptr);
+                           tiles_x, tiles, range_begin, range_end, sorted_ids, records, image, final_T, n_contrib, 1, nullptr, tile_order);
     XAD_HIP_TRY(hipGetLastError());
     return XAD_OK;
 }
@@ -744,18 +807,18 @@ int launch_render_backward(hipStream_t s, int width, int height, const std::uint
                            const std::uint32_t* range_end, const std::uint32_t* sorted_ids, const Record* records,
                            const float* image, const float* target, const float* final_T,
                            const std::uint32_t* n_contrib, float* record_grads, double* loss, int segments,
-                           const float4* segment_state) {
+                           const float4* segment_state, const std::uint32_t* tile_order) {
     const int tiles_x = (width + kTile - 1) / kTile, tiles = tiles_x * ((height + kTile - 1) / kTile);
     XAD_REQUIRE(segments >= 1 && segments <= kMaxSegments && (segments == 1 || segment_state),
                 "splat: a split walk takes up to %d segments and needs its per-segment state", kMaxSegments);
     if (segments > 1)
         hipLaunchKernelGGL(render_backward_kernel<true>, dim3(padded_tile_blocks(tiles) * static_cast<unsigned>(segments)),
                            dim3(kChunk), 0, s, width, height, tiles_x, tiles, range_begin, range_end, sorted_ids, records, image,
-                           target, final_T, n_contrib, record_grads, loss, segments, segment_state);
+                           target, final_T, n_contrib, record_grads, loss, segments, segment_state, tile_order);
     else
         hipLaunchKernelGGL(render_backward_kernel<false>, dim3(padded_tile_blocks(tiles)), dim3(kChunk), 0, s, width, height,
                            tiles_x, tiles, range_begin, range_end, sorted_ids, records, image, target, final_T, n_contrib,
-                           record_grads, loss, 1, nullptr);
+                           record_grads, loss, 1, nullptr, tile_order);
     XAD_HIP_TRY(hipGetLastError());
     return XAD_OK;
 }

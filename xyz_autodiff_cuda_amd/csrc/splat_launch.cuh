@@ -68,12 +68,15 @@ int launch_binning(hipStream_t s, const BinPlan& p, const std::uint32_t* by_dept
                    bool clear_depth_flag);
 int launch_render_forward(hipStream_t s, int width, int height, const std::uint32_t* range_begin,
                           const std::uint32_t* range_end, const std::uint32_t* sorted_ids, const Record* records,
-                          float* image, float* final_T, std::uint32_t* n_contrib, int segments, float4* segment_state);
+                          float* image, float* final_T, std::uint32_t* n_contrib, int segments, float4* segment_state,
+                          std::uint32_t* tile_order);
 int launch_render_backward(hipStream_t s, int width, int height, const std::uint32_t* range_begin,
                            const std::uint32_t* range_end, const std::uint32_t* sorted_ids, const Record* records,
                            const float* image, const float* target, const float* final_T,
                            const std::uint32_t* n_contrib, float* record_grads, double* loss, int segments,
-                           const float4* segment_state);
+                           const float4* segment_state, const std::uint32_t* tile_order);
+// tile_order: 8 * ceil(tiles / 8) words, written by launch_render_forward (the order, longest list first within
+// each XCD's band of tiles, in which the blocks of both kernels take the tiles) and read by launch_render_backward.
 // Pieces a tile's list is cut into for the backward walk (1, 2, 4 or 8: more for images with few tiles);
 // segment_state holds that many float4 per pixel when it is more than one.
 int render_segments(int width, int height);
