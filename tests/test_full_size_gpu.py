@@ -114,13 +114,14 @@ def test_accumulation_16Mi_threads(gpu, oracle, num_slots, strategy):
     assert np.all(got[~touched] == 0.0)
 
 
-def _splat_case(gpu, oracle, G, W, H, scale_px):
+def _splat_case(gpu, oracle, G, W, H, scale_px, opacity_shift=0.0):
     import torch
 
     from xyz_autodiff_cuda_amd import splat
 
     target = splat.synthetic_target(G, W, H, seed=77, scale_px=scale_px, noise=0.02)
     params, depth = splat.synthetic_scene(G, W, H, seed=1234, scale_px=scale_px)
+    params[8] += opacity_shift  # more opaque Gaussians: more pixels reach the 0.99 clamp and the 1e-4 stop
     ctx = splat.SplatContext(W, H, G)
     image, grads, loss = ctx.step(params, depth, target)
     torch.cuda.synchronize()
@@ -182,17 +183,19 @@ def test_splat_exactly_200k_gaussians_2048(gpu, oracle):
     assert 4_000_000 < figures["pairs"] < 12_000_000 and figures["longest_list"] < 5000
 
 
-@pytest.mark.parametrize("W,H,G,scale_px", [
-    (512, 400, 12_000, (1.0, 20.0)),    # 800 tiles: lists walked backward in eight pieces
-    (720, 720, 20_000, (1.0, 24.0)),    # 2025 tiles: four pieces
-    (1000, 1000, 40_000, (1.0, 24.0)),  # 3969 tiles: two pieces
-    (1100, 1100, 40_000, (1.0, 24.0)),  # 4761 tiles: one wavefront walks a tile's whole list
+@pytest.mark.parametrize("W,H,G,scale_px,opacity_shift", [
+    (512, 400, 12_000, (1.0, 20.0), 0.0),    # 800 tiles: lists walked backward in eight pieces
+    (512, 400, 12_000, (1.0, 20.0), 2.5),    # the same with opaque Gaussians: most pixels stop early, pieces start idle
+    (720, 720, 20_000, (1.0, 24.0), 0.0),    # 2025 tiles: four pieces
+    (720, 720, 20_000, (1.0, 24.0), 2.5),
+    (1000, 1000, 40_000, (1.0, 24.0), 0.0),  # 3969 tiles: two pieces
+    (1100, 1100, 40_000, (1.0, 24.0), 0.0),  # 4761 tiles: one wavefront walks a tile's whole list
 ])
-def test_splat_every_way_of_cutting_the_backward_walk(gpu, oracle, W, H, G, scale_px):
+def test_splat_every_way_of_cutting_the_backward_walk(gpu, oracle, W, H, G, scale_px, opacity_shift):
     """The backward walk of a tile's list is cut into more pieces the fewer tiles an image has.  Every
     such layout against the oracle, on scenes dense enough that lists span several pieces and many pixels
     stop early (so that pieces start from a stored state, from the final state, or have nothing to do)."""
-    figures = _splat_case(gpu, oracle, G, W, H, scale_px)
+    figures = _splat_case(gpu, oracle, G, W, H, scale_px, opacity_shift)
     tiles = ((W + 15) // 16) * ((H + 15) // 16)
     assert figures["pairs"] / tiles > 64 and figures["longest_list"] > 128, figures
 
