@@ -123,16 +123,8 @@ __global__ void __launch_bounds__(256) depth_key_kernel(int G, const float* __re
     identity[g] = static_cast<std::uint32_t>(g);
 }
 
-// Blocks are handed to the eight XCDs round-robin; giving each XCD a contiguous
-// band of tiles keeps the records of a Gaussian that spans neighbouring tiles
-// in one L2.
-__device__ __forceinline__ int tile_of_block(int block, int tiles) {
-    constexpr int kXcds = 8;
-    const int per = (tiles + kXcds - 1) / kXcds;
-    const int t = (block % kXcds) * per + block / kXcds;
-    return t;  // may be >= tiles for the padding blocks of the last band
-}
-
+// Blocks are handed to the eight XCDs round-robin; giving each XCD a contiguous band of tiles keeps the
+// records of a Gaussian that spans neighbouring tiles in one L2.
 // Within its band every XCD takes its tiles longest list first: blocks are started in order of their
 // index, and a tile with a long list that starts late leaves the SIMDs around it idle at the end of the
 // launch.  One block per band: a histogram of the list lengths (in units of eight entries) in LDS, a
