@@ -163,6 +163,39 @@ def test_offscreen_and_nonfinite_gaussians(gpu, oracle):
     assert np.all(got["grads"][:, :2] == 0.0)
 
 
+@pytest.mark.parametrize("W,H", [(8, 8), (40, 24), (1100, 1100)])
+def test_a_scene_with_nothing_on_screen(gpu, W, H):
+    """No pair at all: every tile's list is empty, the image is the background, the loss is the target's
+    energy and no gradient is touched (images smaller than a tile, a few tiles, and many tiles)."""
+    G = 50
+    params, depth = random_scene(G, W, H, 3, scale_px=(1.0, 3.0))
+    params[0] = -1000.0 - np.arange(G)  # far off to the left
+    target = np.random.default_rng(2).uniform(0, 1, (H, W, 3)).astype(np.float32)
+    got = _gpu_step(gpu, W, H, params, depth, target)
+    assert got["pairs"] == 0 and got["longest_list"] == 0
+    assert np.all(got["image"] == 0.0) and np.all(got["grads"] == 0.0)
+    assert got["loss"] == pytest.approx(float((target.astype(np.float64) ** 2).sum()), rel=1e-6)
+
+
+def test_host_core_step_and_gpu_step_agree(gpu, oracle):
+    """The step from the library's templates on the host cores and the GPU step, on one scene: the same pairs, the
+    same image to 1e-5, gradients within the tolerance either is held to against the oracle."""
+    from xyz_autodiff_cuda_amd import splat
+
+    G, W, H = 1500, 200, 136
+    params, depth = random_scene(G, W, H, seed=41, scale_px=(1.0, 16.0))
+    target = np.random.default_rng(8).uniform(0, 1, (H, W, 3)).astype(np.float32)
+    got = _gpu_step(gpu, W, H, params, depth, target)
+    host = splat.host_step(params, depth, target, W, H, num_threads=4)
+    assert host["pairs"] == got["pairs"]
+    assert np.abs(host["image"] - got["image"]).max() < 1e-5
+    assert abs(host["loss"] - got["loss"]) <= 1e-6 * got["loss"]
+    o64 = oracle.splat_step(W, H, params, depth, target, np.float64,
+                            rects_in=oracle.splat_step(W, H, params, depth, target, np.float32)["rects"], want_bounds=True)
+    tolerance = 1e-4 * o64["grad_mass"] + o64["grad_bound"] + 1e-30
+    assert (np.abs(host["grads"].astype(np.float64) - got["grads"]) <= 2.0 * tolerance).all()
+
+
 def test_pair_buffers_grow_on_demand(gpu, oracle):
     import torch
 
