@@ -104,7 +104,10 @@ int xad_host_chain_forward_backward_f64(size_t n,
  *                   whole LDS of a CU as fp64 rows for the first ~3000 slots (the
  *                   hottest 32 in several copies), every other slot's contributions
  *                   gathered per wavefront in LDS and written to HBM sixteen rows
- *                   at a time, coalesced.  Every input is read once;
+ *                   at a time, coalesced.  Every input is read once.  That layout
+ *                   suits a law that falls with the slot index; a block whose first
+ *                   1024 slots say otherwise (fewer than half of them own a row)
+ *                   claims 2048 rows on first use instead;
  *   LDS             per-block table of partial sums in LDS, written out once per
  *                   block (the reference's shared-memory pattern,
  *                   tests/test_shared_memory_atomic.cu:29-64, made persistent).

@@ -157,16 +157,22 @@ public:
           replicas_(replicas) {
         hot_ = replicas > 1 ? (hot_rows < 0 || hot_rows > num_slots ? num_slots : hot_rows) : 0;
         hot_stride_ = hot_ | 1;
-        // rows left for the slots themselves once the copies of the hot ones are set aside
-        // (the copies start at an odd row: main_rows_ | 1 must fit in front of them)
-        const int in_front = capacity - (replicas - 1) * hot_stride_;
-        const int left = replicas > 1 ? ((in_front & 1) ? in_front : in_front - 1) : capacity;
-        main_rows_ = tagged_ ? capacity : (num_slots < left ? num_slots : left);
+        main_rows_ = tagged_ ? capacity : main_rows_for(capacity, num_slots, replicas, hot_rows);
         if (hot_ > main_rows_) hot_ = main_rows_;
         copies_base_ = main_rows_ | 1;
         const int copy = static_cast<int>(wave::lane_id() & static_cast<unsigned>(replicas - 1));
         my_copy_ = copy == 0 ? 0 : copies_base_ + (copy - 1) * hot_stride_;
         clear();
+    }
+
+    // Slots that own a row of a table of `capacity` rows that is not tagged: all of them if they fit, else the
+    // first ones, as many as the rows left once the copies of the hot ones are set aside (the copies start at
+    // an odd row: main rows | 1 must fit in front of them).
+    __host__ __device__ static constexpr int main_rows_for(int capacity, int num_slots, int replicas, int hot_rows) {
+        const int hot = replicas > 1 ? (hot_rows < 0 || hot_rows > num_slots ? num_slots : hot_rows) : 0;
+        const int in_front = capacity - (replicas - 1) * (hot | 1);
+        const int left = replicas > 1 ? ((in_front & 1) ? in_front : in_front - 1) : capacity;
+        return num_slots < left ? num_slots : left;
     }
 
     // Rows a table needs for `slots` slots of which the first `hot_rows` are kept in `replicas` copies.

@@ -68,6 +68,27 @@ def test_staged_strategies_match_fp64_sums(gpu, oracle, strategy, num_slots):
     _assert_close(_run(gpu, inputs, slot, num_slots, strategy), ref, 1e-4)
 
 
+@pytest.mark.parametrize("law", ["hot slots last", "uniform", "hot slots in the middle"])
+@pytest.mark.parametrize("num_slots", [3073, 4096, 70000])
+def test_auto_under_laws_whose_low_slots_are_not_the_hot_ones(gpu, oracle, law, num_slots):
+    """Above one table's worth of slots `auto` gives the rows to the first slots, which suits a law that
+    falls with the slot index; a block that sees another law claims its rows on first use instead.  The
+    sums must be right either way (and with blocks deciding differently: the middle law mixes both)."""
+    n = 1_000_003
+    inputs = chain_inputs(n, seed=60 + num_slots % 89)
+    zipf = _zipf_slots(n, num_slots, seed=num_slots + 1)
+    if law == "hot slots last":
+        slot = (num_slots - 1 - zipf).astype(np.int32)
+    elif law == "uniform":
+        slot = np.random.default_rng(num_slots).integers(0, num_slots, n).astype(np.int32)
+    else:
+        # the first half of the threads draw hot slots from the middle, the second half from the front
+        slot = zipf.copy()
+        slot[: n // 2] = (slot[: n // 2] + num_slots // 2) % num_slots
+    ref = _reference(oracle, inputs, slot, num_slots)
+    _assert_close(_run(gpu, inputs, slot, num_slots, "auto"), ref, 1e-4)
+
+
 @pytest.mark.parametrize("strategy", NAIVE)
 @pytest.mark.parametrize("num_slots", [3, 4096])
 def test_naive_global_atomics(gpu, oracle, strategy, num_slots):

@@ -45,6 +45,11 @@ struct AccumulateArgs {
     int claim_rows;
     // slots below this are the ones kept in `replicas` copies (negative: all)
     int hot_rows;
+    // With claim_rows == 0 and a table smaller than the slot count: rows a block falls back to, claimed on
+    // first use, if fewer than half of the first slots it sees are among the ones that own a row (0: never).
+    // The layout by slot index is made for laws whose low slots are the hot ones; under any other law the
+    // hot slots would go through the spill path, one same-address atomic after the other.
+    int fallback_rows;
 };
 
 // Which part a block serves, the rows of its table and where they live in the global array.
@@ -65,13 +70,38 @@ template <Strategy S, int Peel, typename TableT, bool Spill = false>
 __global__ void __launch_bounds__(kBlock) accumulate_kernel(AccumulateArgs a) {
     extern __shared__ __attribute__((aligned(16))) float lds[];
     const Part part(a);
-    BlockAccumulator<float, kWidth, S, Peel, 4, TableT, Spill> acc(lds, a.capacity, a.grads + part.index * kWidth,
-                                                                   part.rows, part.parts * kWidth, a.replicas,
-                                                                   a.claim_rows != 0, a.hot_rows);
-    if constexpr (Spill) acc.use_spill_staging(reinterpret_cast<char*>(lds) + a.spill_offset);
-
     const std::size_t begin = static_cast<std::size_t>(blockIdx.x >> a.part_shift) * a.per_block;
     const std::size_t end = begin + a.per_block < a.n ? begin + a.per_block : a.n;
+    using Acc = BlockAccumulator<float, kWidth, S, Peel, 4, TableT, Spill>;
+    if (a.fallback_rows > 0) {  // the same for every block
+        // the block's first slots as a sample of the law: who would find a row of its own?
+        const std::size_t i = begin + threadIdx.x;
+        const int sample = i < end ? part.row_of(a.slot[i], a) : -1;
+        const int owners = Acc::main_rows_for(a.capacity, part.rows, a.replicas, a.hot_rows);
+        // counted in the first two words of the table's memory, which the accumulator clears afterwards
+        int* count = reinterpret_cast<int*>(lds);
+        if (threadIdx.x < 2) count[threadIdx.x] = 0;
+        __syncthreads();
+        const int seen_here = __builtin_popcountll(xyz_autodiff::accumulate::wave::ballot(sample >= 0));
+        const int served_here = __builtin_popcountll(xyz_autodiff::accumulate::wave::ballot(sample >= 0 && sample < owners));
+        if (xyz_autodiff::accumulate::wave::lane_id() == 0) {
+            atomicAdd(count + 0, seen_here);
+            atomicAdd(count + 1, served_here);
+        }
+        __syncthreads();
+        const int seen = count[0], served = count[1];
+        __syncthreads();
+        if (2 * served < seen) {
+            a.capacity = a.fallback_rows;
+            a.replicas = 1;
+            a.claim_rows = 1;
+            a.hot_rows = -1;
+        }
+    }
+    Acc acc(lds, a.capacity, a.grads + part.index * kWidth, part.rows, part.parts * kWidth, a.replicas, a.claim_rows != 0,
+            a.hot_rows);
+    if constexpr (Spill) acc.use_spill_staging(reinterpret_cast<char*>(lds) + a.spill_offset);
+
     // The inputs of the next trip are requested before the arithmetic of this one, so that a lane has
     // two trips' worth of loads in flight instead of waiting for memory twice per trip (slot, then inputs).
     struct Inputs {
@@ -205,7 +235,7 @@ extern "C" int xad_accumulate_chain_gradients_f32(int strategy, std::size_t n, c
                                                   void* stream) {
     const char* who = "xad_accumulate_chain_gradients_f32";
     if (n == 0) return XAD_OK;
-    AccumulateArgs a{{sx, sy, theta, o, px, py}, slot, grads, n, 0, num_slots, 0, 0, 0, 1, 1, -1};
+    AccumulateArgs a{{sx, sy, theta, o, px, py}, slot, grads, n, 0, num_slots, 0, 0, 0, 1, 1, -1, 0};
     for (int k = 0; k < 6; ++k) XAD_REQUIRE(a.in[k], "%s: input array %d is null", who, k);
     XAD_REQUIRE(slot && grads, "%s: slot or grads is null", who);
     XAD_REQUIRE(num_slots > 0, "%s: num_slots must be positive, got %d", who, num_slots);
@@ -229,6 +259,7 @@ extern "C" int xad_accumulate_chain_gradients_f32(int strategy, std::size_t n, c
             // from the other slots cost more (262 144 slots: 0.241 ms with 4 copies, 0.257 with 8, 0.265 with none).
             a.replicas = num_slots <= 32768 ? 8 : 4;
             a.hot_rows = 32;
+            a.fallback_rows = 2048;  // with their tags the most fp64 rows in a power of two that fit
             a.spill_offset = static_cast<unsigned>(static_cast<std::size_t>(rows) * kRowBytes);
             return launch(accumulate_kernel<Strategy::LdsAtomics, 0, double, true>, a, a.spill_offset + kSpillBytes, 1, stream);
         }
