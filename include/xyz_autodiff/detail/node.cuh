@@ -23,10 +23,12 @@
 // between the forward passes of two such roots.
 //
 // A forward() that no backward() follows leaves visits registered.  Every node
-// remembers whether it has registered visits that were never released, and the
-// next forward() of that node first withdraws exactly those (recursively, through
-// operands whose count drops to zero), so forward(); forward(); backward() works
-// and never disturbs the visits of another root.
+// remembers that it holds a visit on each of its operands, and its next
+// evaluation walks them again without registering a second one: the operands
+// are evaluated afresh (a forward() always recomputes what lies below it), the
+// counts stay what they were, so forward(); forward(); backward() works and
+// never disturbs the visits of another root.  There is no separate pass that
+// takes visits back: one walk, one call per edge, nothing recursive besides it.
 //
 // All counts are compile-time constants once the graph is inlined, so none of
 // this survives into the ISA: it only decides which calls are emitted.
@@ -49,30 +51,18 @@ namespace xyz_autodiff {
 namespace detail {
 
 template <typename X>
-concept HasVisitProtocol = requires(X x) {
-    x.xad_visit();
-    x.xad_unvisit();
-};
+concept HasVisitProtocol = requires(X x, bool held) { x.xad_visit(held); };
 
-// Takes back one visit that will never be released (its consumer is about to
-// be evaluated again).  A node of the three-call protocol can only be told
-// that one consumer is gone.
+// A consumer reaches one operand during its evaluation.  `held` says that the
+// consumer still holds the visit of an earlier evaluation that no backward
+// followed: the operand is then evaluated again and not counted again.
 template <typename X>
-XAD_INLINE void unvisit_operand(X& x) {
+XAD_INLINE void visit_operand(X& x, bool held) {
     if constexpr (HasVisitProtocol<X>) {
-        x.xad_unvisit();
-    } else if constexpr (OperationNode<X>) {
-        (void)x.decrement_ref_count_and_check();
-    }
-}
-
-template <typename X>
-XAD_INLINE void visit_operand(X& x) {
-    if constexpr (HasVisitProtocol<X>) {
-        x.xad_visit();
+        x.xad_visit(held);
     } else if constexpr (OperationNode<X>) {
         x.forward();
-        x.increment_ref_count();
+        if (!held) x.increment_ref_count();
     }
 }
 
@@ -144,26 +134,23 @@ public:
 
     // A moved node starts with no registered consumers.
     XAD_HD Node(Node&& other) noexcept
-        : logic_(other.logic_), in_(other.in_), out_(other.out_), pending_(0), owes_release_(false) {}
+        : logic_(other.logic_), in_(other.in_), out_(other.out_), pending_(0), holds_visits_(false) {}
 
     // Construction records the operands; nothing is evaluated until forward().
     XAD_HD Node(const Logic& logic, Ins&... ins)
-        : logic_(logic), in_{ins...}, out_(), pending_(0), owes_release_(false) {}
+        : logic_(logic), in_{ins...}, out_(), pending_(0), holds_visits_(false) {}
 
     // ---- evaluation -------------------------------------------------------
 
     // Evaluates the whole sub-graph below this node, each node once.
-    XAD_INLINE void forward() {
-        withdraw();
-        evaluate();
-    }
+    XAD_INLINE void forward() { evaluate(); }
 
     // Propagates this node's gradient to its operands and fires every operand
     // whose last consumer this was.
     XAD_INLINE void backward() {
         const output_type& out = out_;
         in_.all([&](auto&... xs) { logic_.backward(out, xs...); });
-        owes_release_ = false;
+        holds_visits_ = false;
         in_.each([](auto& x) { release_operand(x); });
     }
 
@@ -174,7 +161,7 @@ public:
     // is passed twice to one node is perturbed (and credited) once per slot.
     XAD_INLINE void backward_numerical(const value_type delta = value_type(1e-5)) {
         in_.each([&](auto& x) { this->perturb(x, delta); });
-        owes_release_ = false;
+        holds_visits_ = false;
         in_.each([&](auto& x) { release_operand_numerical(x, delta); });
     }
 
@@ -197,11 +184,12 @@ public:
     // A release without a matching visit is ignored rather than wrapping the count.
     XAD_INLINE bool decrement_ref_count_and_check() { return pending_ != 0 && --pending_ == 0; }
 
-    XAD_INLINE void xad_visit() {
-        if (pending_++ == 0) evaluate();
-    }
-    XAD_INLINE void xad_unvisit() {
-        if (pending_ != 0 && --pending_ == 0) withdraw();
+    // The first visit of a pass evaluates the node, later ones only count; a
+    // consumer that walks its operands a second time evaluates without counting.
+    XAD_INLINE void xad_visit(bool held) {
+        const bool fresh = pending_ == 0;
+        if (!held) ++pending_;
+        if (held || fresh) evaluate();
     }
 
     // ---- the node as a differentiable variable ---------------------------
@@ -224,18 +212,11 @@ private:
     // Operands first, then this node.  The node's gradient restarts from zero
     // with every evaluation, so a graph object can be run any number of times.
     XAD_INLINE void evaluate() {
-        in_.each([](auto& x) { visit_operand(x); });
-        owes_release_ = true;
+        const bool held = holds_visits_;
+        in_.each([held](auto& x) { visit_operand(x, held); });
+        holds_visits_ = true;
         out_.zero_grad();
         in_.all([&](const auto&... xs) { logic_.forward(out_, xs...); });
-    }
-
-    // Takes back the visits of an evaluation of this node that no backward followed.
-    XAD_INLINE void withdraw() {
-        if (owes_release_) {
-            owes_release_ = false;
-            in_.each([](auto& x) { unvisit_operand(x); });
-        }
     }
 
     XAD_INLINE void seed() {
@@ -267,7 +248,7 @@ private:
     Operands<Ins...> in_;
     output_type out_;
     std::uint8_t pending_;
-    bool owes_release_;  // visits registered with the operands and not yet released
+    bool holds_visits_;  // one visit registered with every operand and not yet released
 };
 
 }  // namespace detail

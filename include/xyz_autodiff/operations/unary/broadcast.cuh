@@ -24,7 +24,7 @@ public:
     using value_type = typename Input::value_type;
     static constexpr std::size_t size = OutputSize;
 
-    XAD_HD explicit BroadcastOperator(Input& input) : source_(input), pending_(0), owes_release_(false) {}
+    XAD_HD explicit BroadcastOperator(Input& input) : source_(input), pending_(0), holds_visit_(false) {}
 
     // ---- differentiable-variable face ------------------------------------
     XAD_INLINE const value_type& operator[](std::size_t) const { return source_[0]; }
@@ -34,16 +34,13 @@ public:
     XAD_INLINE void zero_grad() { source_.zero_grad(); }
 
     // ---- node face: only traversal, no arithmetic --------------------------
-    XAD_INLINE void forward() {
-        withdraw();
-        evaluate();
-    }
+    XAD_INLINE void forward() { evaluate(); }
     XAD_INLINE void backward() {
-        owes_release_ = false;
+        holds_visit_ = false;
         detail::release_operand(source_);
     }
     XAD_INLINE void backward_numerical(value_type delta = value_type(1e-5)) {
-        owes_release_ = false;
+        holds_visit_ = false;
         detail::release_operand_numerical(source_, delta);
     }
     XAD_INLINE void run() {
@@ -57,29 +54,22 @@ public:
 
     XAD_INLINE void increment_ref_count() const { ++pending_; }
     XAD_INLINE bool decrement_ref_count_and_check() const { return pending_ != 0 && --pending_ == 0; }
-    XAD_INLINE void xad_visit() {
-        if (pending_++ == 0) evaluate();
-    }
-    XAD_INLINE void xad_unvisit() {
-        if (pending_ != 0 && --pending_ == 0) withdraw();
+    XAD_INLINE void xad_visit(bool held) {
+        const bool fresh = pending_ == 0;
+        if (!held) ++pending_;
+        if (held || fresh) evaluate();
     }
 
 private:
+    // a second walk without a backward in between does not count again (see detail/node.cuh)
     XAD_INLINE void evaluate() {
-        detail::visit_operand(source_);
-        owes_release_ = true;
-    }
-    // takes back the visit of an evaluation that no backward followed (see detail/node.cuh)
-    XAD_INLINE void withdraw() {
-        if (owes_release_) {
-            owes_release_ = false;
-            detail::unvisit_operand(source_);
-        }
+        detail::visit_operand(source_, holds_visit_);
+        holds_visit_ = true;
     }
 
     Input& source_;
     mutable std::uint8_t pending_;
-    bool owes_release_;
+    bool holds_visit_;
 };
 
 template <std::size_t OutputSize, typename Input>

@@ -510,6 +510,22 @@ XAD_HD inline int run_case(int id, double* out) {
                 abandoned.backward();
                 put(x.grad(0));  // (2 s - 1) s
             }
+            {   // a node with two consumers inside one graph, walked twice before the backward pass:
+                //   y = s + s^2 through a broadcast, s = exp(x); the second walk sees x = 0.25 and counts nothing twice
+                Variable<1, double> x(0.5);
+                auto s = op::exp(x);
+                auto s2 = op::squared(s);
+                auto y = s + s2;
+                auto wide = op::broadcast<3>(y);
+                auto total = op::sum(wide);
+                total.forward();
+                put(total[0]);  // 3 (e^0.5 + e)
+                x[0] = 0.25;
+                total.forward();
+                total.add_grad(0, 1.0);
+                total.backward();
+                put(total[0]); put(x.grad(0));  // 3 (e^0.25 + e^0.5), 3 (e^0.25 + 2 e^0.5)
+            }
             break;
         }
         default:

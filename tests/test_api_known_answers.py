@@ -31,7 +31,8 @@ EXPECTED = {
     # node operands: e^0.6 - 0.3, 2 e^0.6 - 1; a ternary node consumed twice: 3.5 + 3.5^2, 8 (b, a, 1)
     16: [1.0, -7.0] + [0.5, 3.0, 1.5, -2.0, 1.0, 1.0] * 2 + [E ** 0.6 - 0.3, 2 * E ** 0.6 - 1] + [15.75, 12.0, 16.0, 8.0],
     # roots sharing a node: 0 until the last root has released it, then (2 s - 1) s with s = e^0.5
-    17: [0.0, -E ** 0.5, E, (2 * E ** 0.5 - 1) * E ** 0.5] + [E ** 0.5, 2 * E ** 0.5] + [0.0, (2 * E ** 0.5 - 1) * E ** 0.5],
+    17: [0.0, -E ** 0.5, E, (2 * E ** 0.5 - 1) * E ** 0.5] + [E ** 0.5, 2 * E ** 0.5] + [0.0, (2 * E ** 0.5 - 1) * E ** 0.5]
+        + [3 * (E ** 0.5 + E), 3 * (E ** 0.25 + E ** 0.5), 3 * (E ** 0.25 + 2 * E ** 0.5)],
 }
 
 
