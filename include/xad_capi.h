@@ -180,11 +180,13 @@ int xad_accumulate_chain_gradients_f32(int strategy, size_t n,
  * depths change all the time sets XAD_SPLAT_DEPTH_EVERY_STEP (the order is
  * recomputed by every call, on the device).  In both modes a step with
  * loss_out == NULL only queues work.  What such a call cannot report itself is
- * reported by the next call that waits (a step with loss_out, xad_splat_get_stats):
- * XAD_ERR_INCOMPLETE if a step produced more pairs than the lists held (its image
- * and gradients lack the pairs that did not fit; the lists are enlarged at that
- * point), XAD_ERR_INVALID_ARGUMENT if a depth changed under the static promise.
- * The outputs of the call that returns such a status are themselves complete.
+ * reported by the next call that waits (a step with loss_out, xad_splat_get_stats,
+ * xad_splat_get_lists): XAD_ERR_INCOMPLETE if a step produced more pairs than the
+ * lists held (its image and gradients lack the pairs that did not fit; the lists
+ * are enlarged at that point), XAD_ERR_INVALID_ARGUMENT if a depth changed under
+ * the static promise.  The outputs of a step that returns such a status are
+ * themselves complete.  A caller that must not act on incomplete gradients without
+ * waiting for them gates its update on the device: see xad_splat_overflow_word.
  *
  * Recording.  In XAD_SPLAT_DEPTH_STATIC mode, after a step with loss_out has
  * returned (the lists are sized then), xad_splat_step with loss_out == NULL is a
@@ -198,7 +200,10 @@ typedef struct xad_splat_context xad_splat_context;
 int xad_splat_create(int width, int height, int num_gaussians, size_t pair_capacity_hint,
                      xad_splat_context** out);
 void xad_splat_destroy(xad_splat_context* ctx);
-/* Render only. */
+/* Render only.  In XAD_SPLAT_DEPTH_CHECKED mode the call waits for the binning
+ * anyway and enlarges the lists itself when the scene has outgrown them, so its
+ * image is always complete; in the other two modes what is said above of calls
+ * that only queue work applies. */
 int xad_splat_forward(xad_splat_context* ctx, const float* params, const float* depth,
                       float* image, void* stream);
 /* Render, loss and gradients.  loss_out (host, may be NULL) receives the sum of
@@ -225,6 +230,13 @@ int xad_splat_get_stats(xad_splat_context* ctx, uint64_t* pairs, uint32_t* longe
  * entries, at least the pair count.  Waits for the device. */
 int xad_splat_get_lists(xad_splat_context* ctx, uint32_t* range_begin, uint32_t* range_end,
                         uint32_t* gaussians, size_t capacity);
+/* Device address of one 32-bit word that is zero as long as every step since the
+ * host last looked fitted the lists, and not zero from the binning of the first
+ * step that did not until a call that waits has enlarged them.  Work queued behind
+ * a step on the same stream may read it to decide on the device whether to use
+ * that step's gradients (xad_adam_step_gated_f32).  Valid for the context's life.
+ * No counterpart in the reference, whose one kernel needs no lists. */
+int xad_splat_overflow_word(xad_splat_context* ctx, const uint32_t** device_word);
 /* The same step on the host cores, every pointer host memory: the CPU figure the
  * GPU step is reported beside.  Tiles are dealt to num_threads threads (0: one per
  * hardware thread); every (pixel, Gaussian) pair builds the renderer's per-pair
@@ -246,6 +258,16 @@ int xad_host_splat_step_f32(int width, int height, int num_gaussians, const floa
 int xad_adam_step_f32(size_t n, int rows, float* params, const float* grads, float* m, float* v,
                       const float* row_learning_rates, float beta1, float beta2, float eps,
                       int iteration, void* stream);
+/* The same update, decided on the device: the kernel first reads *hold_if_nonzero
+ * (device) and, if it is not zero, changes nothing and adds one to *held_count
+ * (device, may be NULL).  For training loops that do not wait for the device
+ * between the gradients and the update (the reference's loop computes all
+ * gradients, then steps, gaussian_splatting_training.cu:127-160: an update never
+ * sees partial gradients there). */
+int xad_adam_step_gated_f32(size_t n, int rows, float* params, const float* grads, float* m, float* v,
+                            const float* row_learning_rates, float beta1, float beta2, float eps,
+                            int iteration, const uint32_t* hold_if_nonzero, uint32_t* held_count,
+                            void* stream);
 
 /* ---------------------------------------------------------------------------
  * Splatting trainer front-end: configuration, image files, training loop,
@@ -318,11 +340,15 @@ int xad_trainer_create(const xad_training_config* config, int width, int height,
 void xad_trainer_destroy(xad_trainer* trainer);
 /* Runs `iterations` iterations.  loss_out (host, may be NULL) receives the sum
  * of squared errors of the last iteration's rendering, taken before its update.
- * Only an iteration that reports its loss waits for the device.  Returns
- * XAD_ERR_INCOMPLETE, with every iteration run and loss_out set, if the tile lists
- * outgrew their buffers in an iteration since the last reported loss (that
- * iteration's gradients lacked contributions; the buffers have been enlarged). */
+ * Only an iteration that reports its loss waits for the device (and the host
+ * stays at most 32 iterations ahead of it).  No update is ever applied to
+ * gradients from tile lists that had outgrown their buffers: such an update is
+ * withheld on the device, and when the host next looks the buffers are enlarged
+ * and the iterations since then are run again with their own step numbers, so
+ * the result is that of a run whose buffers were ample from the start. */
 int xad_trainer_run(xad_trainer* trainer, int iterations, double* loss_out);
+/* Iterations that had to be run a second time for that reason, over the trainer's life. */
+long long xad_trainer_repeated_iterations(const xad_trainer* trainer);
 /* Iterations completed so far (continues from the checkpoint after a load). */
 int xad_trainer_iteration(const xad_trainer* trainer);
 /* The last rendering (zeros before the first iteration), to host memory. */

@@ -313,6 +313,86 @@ def test_full_size_config5_properties(gpu):
     ctx2.close()
 
 
+def test_the_getters_report_and_settle_an_overflow_too(gpu, oracle, xad):
+    """xad_splat_get_stats and xad_splat_get_lists wait for the device, so they are calls that report what a
+    step that did not wait has left behind, and enlarge the lists."""
+    import torch
+
+    from xyz_autodiff_cuda_amd import splat
+
+    G, W, H = 600, 256, 256
+    small, depth = random_scene(G, W, H, seed=5, scale_px=(0.5, 1.0))
+    large = small.copy()
+    large[2:4] += np.log(30.0)
+    target = np.zeros((H, W, 3), np.float32)
+    d, t = torch.from_numpy(depth).to(gpu), torch.from_numpy(target).to(gpu)
+    ref = oracle.splat_step(W, H, large, depth, target, np.float32)
+    for getter in ("stats", "lists"):
+        ctx = splat.SplatContext(W, H, G, pair_capacity_hint=4000, depth_mode="static")
+        ctx.step(torch.from_numpy(small).to(gpu), d, t)
+        ctx.step(torch.from_numpy(large).to(gpu), d, t, want_loss=False)
+        with pytest.raises(xad.XadError, match="incomplete"):
+            getattr(ctx, getter)()
+        # settled: the same step fits now without anybody waiting for it, and the getters answer
+        image, _, _ = ctx.step(torch.from_numpy(large).to(gpu), d, t, want_loss=False)
+        assert ctx.stats()["pairs"] == ref["pairs"]
+        begin, end, ids = ctx.lists()
+        assert int((end - begin).sum()) == ref["pairs"] == ids.size
+        assert np.abs(image.cpu().numpy() - ref["image"]).max() < 5e-5
+        ctx.close()
+
+
+def test_forward_only_calls_enlarge_the_lists_themselves(gpu, oracle):
+    """In the default depth mode a forward call waits for the binning anyway: a scene that has outgrown the lists
+    is binned again into larger ones before anything is composited, also when no call ever asks for a loss."""
+    import torch
+
+    from xyz_autodiff_cuda_amd import splat
+
+    G, W, H = 600, 256, 256
+    small, depth = random_scene(G, W, H, seed=5, scale_px=(0.5, 1.0))
+    target = np.zeros((H, W, 3), np.float32)
+    d = torch.from_numpy(depth).to(gpu)
+    ctx = splat.SplatContext(W, H, G, pair_capacity_hint=4000)
+    ctx.forward(torch.from_numpy(small).to(gpu), d)
+    for widen in (6.0, 30.0, 90.0):  # each many times the pairs of the one before
+        scene = small.copy()
+        scene[2:4] += np.log(widen)
+        image = ctx.forward(torch.from_numpy(scene).to(gpu), d)
+        torch.cuda.synchronize()
+        ref = oracle.splat_step(W, H, scene, depth, target, np.float32)
+        assert np.abs(image.cpu().numpy() - ref["image"]).max() < 5e-5, widen
+        assert ctx.stats()["pairs"] == ref["pairs"], widen
+    ctx.close()
+
+
+def test_gated_adam_holds_the_update_when_told_to(gpu, oracle):
+    import torch
+
+    from xyz_autodiff_cuda_amd import splat
+
+    rows, n = 9, 1000
+    r = np.random.default_rng(5)
+    p0 = r.normal(0, 1, (rows, n)).astype(np.float32)
+    g = torch.from_numpy(r.normal(0, 2, (rows, n)).astype(np.float32)).to(gpu)
+    gate = torch.zeros(1, dtype=torch.int32, device=gpu)
+    held = torch.zeros(1, dtype=torch.int32, device=gpu)
+    plain = [torch.from_numpy(p0.copy()).to(gpu), torch.zeros(rows, n, device=gpu), torch.zeros(rows, n, device=gpu)]
+    gated = [x.clone() for x in plain]
+    splat.adam_step(plain[0], g, plain[1], plain[2], 1e-2, 1)
+    splat.adam_step(gated[0], g, gated[1], gated[2], 1e-2, 1, hold_if_nonzero=gate, held_count=held)
+    assert all(torch.equal(a, b) for a, b in zip(plain, gated)) and int(held) == 0
+    gate.fill_(7)
+    before = [x.clone() for x in gated]
+    for _ in range(3):
+        splat.adam_step(gated[0], g, gated[1], gated[2], 1e-2, 2, hold_if_nonzero=gate, held_count=held)
+    assert all(torch.equal(a, b) for a, b in zip(before, gated)) and int(held) == 3
+    gate.zero_()
+    splat.adam_step(plain[0], g, plain[1], plain[2], 1e-2, 2)
+    splat.adam_step(gated[0], g, gated[1], gated[2], 1e-2, 2, hold_if_nonzero=gate, held_count=held)
+    assert all(torch.equal(a, b) for a, b in zip(plain, gated)) and int(held) == 3
+
+
 # ---- the tile lists themselves (integer work: must equal what the oracle's rectangles and the depths imply) ----
 
 def _expected_lists(rects, depth, tiles_x, tiles_y):
@@ -487,8 +567,11 @@ def test_overflow_in_a_step_that_does_not_wait_is_reported_later(gpu, oracle, xa
     ctx.step(torch.from_numpy(small).to(gpu), d, t)  # sized for the small scene
     few = ctx.stats()["pairs"]
     ctx.step(torch.from_numpy(large).to(gpu), d, t, want_loss=False)  # does not fit, and nobody is told yet
-    with pytest.raises(xad.XadError, match="incomplete"):
-        ctx.step(torch.from_numpy(small).to(gpu), d, t)
+    # the next step that waits says so; its own outputs are complete and are handed out
+    with pytest.warns(RuntimeWarning, match="incomplete"):
+        image, _, loss = ctx.step(torch.from_numpy(small).to(gpu), d, t)
+    ref_small = oracle.splat_step(W, H, small, depth, target, np.float32)
+    assert np.abs(image.cpu().numpy() - ref_small["image"]).max() < 1e-5 and abs(loss - ref_small["loss"]) <= 1e-6 * ref_small["loss"]
     image, grads, loss = ctx.step(torch.from_numpy(large).to(gpu), d, t)  # the lists were enlarged: complete now
     ref = oracle.splat_step(W, H, large, depth, target, np.float32)
     assert ctx.stats()["pairs"] == ref["pairs"] > 4 * few
@@ -502,3 +585,83 @@ def test_overflow_in_a_step_that_does_not_wait_is_reported_later(gpu, oracle, xa
     assert np.abs(image2.cpu().numpy() - ref["image"]).max() < 5e-5 and abs(loss2 - ref["loss"]) <= 1e-5 * ref["loss"] + 1e-9
     ctx.close()
     ctx2.close()
+
+
+def test_the_getters_report_and_settle_an_overflow_too(gpu, oracle, xad):
+    """xad_splat_get_stats and xad_splat_get_lists wait for the device, so they are calls that report what a
+    step that did not wait has left behind, and enlarge the lists."""
+    import torch
+
+    from xyz_autodiff_cuda_amd import splat
+
+    G, W, H = 600, 256, 256
+    small, depth = random_scene(G, W, H, seed=5, scale_px=(0.5, 1.0))
+    large = small.copy()
+    large[2:4] += np.log(30.0)
+    target = np.zeros((H, W, 3), np.float32)
+    d, t = torch.from_numpy(depth).to(gpu), torch.from_numpy(target).to(gpu)
+    ref = oracle.splat_step(W, H, large, depth, target, np.float32)
+    for getter in ("stats", "lists"):
+        ctx = splat.SplatContext(W, H, G, pair_capacity_hint=4000, depth_mode="static")
+        ctx.step(torch.from_numpy(small).to(gpu), d, t)
+        ctx.step(torch.from_numpy(large).to(gpu), d, t, want_loss=False)
+        with pytest.raises(xad.XadError, match="incomplete"):
+            getattr(ctx, getter)()
+        # settled: the same step fits now without anybody waiting for it, and the getters answer
+        image, _, _ = ctx.step(torch.from_numpy(large).to(gpu), d, t, want_loss=False)
+        assert ctx.stats()["pairs"] == ref["pairs"]
+        begin, end, ids = ctx.lists()
+        assert int((end - begin).sum()) == ref["pairs"] == ids.size
+        assert np.abs(image.cpu().numpy() - ref["image"]).max() < 5e-5
+        ctx.close()
+
+
+def test_forward_only_calls_enlarge_the_lists_themselves(gpu, oracle):
+    """In the default depth mode a forward call waits for the binning anyway: a scene that has outgrown the lists
+    is binned again into larger ones before anything is composited, also when no call ever asks for a loss."""
+    import torch
+
+    from xyz_autodiff_cuda_amd import splat
+
+    G, W, H = 600, 256, 256
+    small, depth = random_scene(G, W, H, seed=5, scale_px=(0.5, 1.0))
+    target = np.zeros((H, W, 3), np.float32)
+    d = torch.from_numpy(depth).to(gpu)
+    ctx = splat.SplatContext(W, H, G, pair_capacity_hint=4000)
+    ctx.forward(torch.from_numpy(small).to(gpu), d)
+    for widen in (6.0, 30.0, 90.0):  # each many times the pairs of the one before
+        scene = small.copy()
+        scene[2:4] += np.log(widen)
+        image = ctx.forward(torch.from_numpy(scene).to(gpu), d)
+        torch.cuda.synchronize()
+        ref = oracle.splat_step(W, H, scene, depth, target, np.float32)
+        assert np.abs(image.cpu().numpy() - ref["image"]).max() < 5e-5, widen
+        assert ctx.stats()["pairs"] == ref["pairs"], widen
+    ctx.close()
+
+
+def test_gated_adam_holds_the_update_when_told_to(gpu, oracle):
+    import torch
+
+    from xyz_autodiff_cuda_amd import splat
+
+    rows, n = 9, 1000
+    r = np.random.default_rng(5)
+    p0 = r.normal(0, 1, (rows, n)).astype(np.float32)
+    g = torch.from_numpy(r.normal(0, 2, (rows, n)).astype(np.float32)).to(gpu)
+    gate = torch.zeros(1, dtype=torch.int32, device=gpu)
+    held = torch.zeros(1, dtype=torch.int32, device=gpu)
+    plain = [torch.from_numpy(p0.copy()).to(gpu), torch.zeros(rows, n, device=gpu), torch.zeros(rows, n, device=gpu)]
+    gated = [x.clone() for x in plain]
+    splat.adam_step(plain[0], g, plain[1], plain[2], 1e-2, 1)
+    splat.adam_step(gated[0], g, gated[1], gated[2], 1e-2, 1, hold_if_nonzero=gate, held_count=held)
+    assert all(torch.equal(a, b) for a, b in zip(plain, gated)) and int(held) == 0
+    gate.fill_(7)
+    before = [x.clone() for x in gated]
+    for _ in range(3):
+        splat.adam_step(gated[0], g, gated[1], gated[2], 1e-2, 2, hold_if_nonzero=gate, held_count=held)
+    assert all(torch.equal(a, b) for a, b in zip(before, gated)) and int(held) == 3
+    gate.zero_()
+    splat.adam_step(plain[0], g, plain[1], plain[2], 1e-2, 2)
+    splat.adam_step(gated[0], g, gated[1], gated[2], 1e-2, 2, hold_if_nonzero=gate, held_count=held)
+    assert all(torch.equal(a, b) for a, b in zip(plain, gated)) and int(held) == 3

@@ -89,30 +89,151 @@ def test_training_fits_the_test_pattern(gpu):
     t.close()
 
 
-def test_lists_that_outgrow_their_buffers_during_a_run_are_reported_and_the_run_goes_on(gpu):
-    """Iterations that do not report a loss never wait for the device, so a run whose Gaussians have grown
-    outgrows the tile lists' buffers unnoticed.  The run must finish, say so once its last iteration reads the
-    device's report, and work normally afterwards with the enlarged buffers."""
-    W = H = 256
-    target = trainer.test_pattern(W, H)
-    t = trainer.Trainer(_config(num_gaussians=4000), target)
-    t.run(2)  # sizes the buffers for the initial Gaussians (a few pixels across)
-    params = t.state()["params"]
-    params[2:4] += 2.0  # seven times as wide: about twenty times the pairs
-    t.set_params(params)
-    with pytest.warns(RuntimeWarning, match="outgrown their buffers"):
-        loss = t.run(8)
-    assert t.iteration == 10 and np.isfinite(loss)
+def _grown_state(W, H, G, target):
+    """State of a short run whose Gaussians were then made seven times as wide (about twenty times the pairs)."""
+    t = trainer.Trainer(_config(num_gaussians=G), target)
+    t.run(2)
     state = t.state()
-    assert all(np.isfinite(v).all() for v in state.values() if isinstance(v, np.ndarray))
-    # the report has been taken and the buffers fit again: a rendering with every contribution
+    t.close()
+    state["params"][2:4] += 2.0
+    return state
+
+
+@pytest.mark.parametrize("iterations,loss_every", [(40, 0), (24, 6), (7, 1)])
+def test_a_run_whose_lists_outgrow_their_buffers_equals_a_run_with_ample_buffers(gpu, iterations, loss_every):
+    """Iterations that do not report a loss never wait for the device, so nobody sees that the tile lists of a
+    scene that has grown no longer fit.  No update may use such gradients (the loop of the reference computes all
+    gradients, then steps: gaussian_splatting_training.cu:127-160): the updates are withheld on the device, and the
+    iterations are run again once the host has looked.  The result must be that of a run whose buffers were ample
+    from the start, step numbers included."""
+    W = H = 256
+    G = 4000
+    target = trainer.test_pattern(W, H)
+    state = _grown_state(W, H, G, target)
+
+    def run(t):
+        losses = []
+        if loss_every:
+            for _ in range(iterations // loss_every):
+                losses.append(t.run(loss_every))
+            if iterations % loss_every:
+                losses.append(t.run(iterations % loss_every))
+        else:
+            t.run(iterations, want_loss=False)
+            losses.append(t.run(1))
+        return losses
+
+    tight = trainer.Trainer(_config(num_gaussians=G), target)
+    tight.run(2)  # its buffers are sized for the initial Gaussians, a few pixels across
+    tight.set_params(state["params"])
+    ample = trainer.Trainer(_config(num_gaussians=G), target)
+    ample.set_params(state["params"])
+    ample.run(2)  # its buffers are sized for the wide ones
+    # the same starting point for both: the wide scene, iteration 2, the moments of `tight`
+    import tempfile
+
+    with tempfile.TemporaryDirectory() as tmp:
+        path = os.path.join(tmp, "start.ckpt")
+        tight.save_checkpoint(path)
+        ample.load_checkpoint(path)
+    start = tight.iteration
     import warnings
 
     with warnings.catch_warnings():
         warnings.simplefilter("error")
-        again = t.run(1)
-    assert np.isfinite(again) and np.mean((t.image() - target) ** 2) * 3 * W * H == pytest.approx(again, rel=1e-3)
+        loss_tight = run(tight)
+        loss_ample = run(ample)
+    # (a run that reports every iteration's loss waits every time: the step itself is run again, no iteration is)
+    assert (tight.repeated_iterations > 0) == (loss_every != 1) and ample.repeated_iterations == 0
+    assert tight.iteration == ample.iteration == start + iterations + (0 if loss_every else 1)
+    a, b = tight.state(), ample.state()
+    for x, y in zip(loss_tight, loss_ample):
+        assert abs(x - y) <= 1e-3 * abs(y), (loss_tight, loss_ample)
+    for row in range(9):
+        # the two runs differ by the order of the atomic sums only: nearly every element agrees to a small part
+        # of a step; an element whose gradient is rounding noise around zero may move the other way in some
+        # iteration (Adam moves by about lr whatever the gradient's size)
+        off = np.abs(a["params"][row] - b["params"][row]) / ROW_LRS[row]
+        assert np.quantile(off, 0.99) <= 0.02 * iterations and off.max() <= 2.0 * iterations, (row, np.quantile(off, 0.99), off.max())
+        scale_m = np.abs(b["m"][row]).max() + 1e-20
+        assert np.quantile(np.abs(a["m"][row] - b["m"][row]), 0.99) <= 1e-2 * scale_m, row
+    np.testing.assert_array_equal(a["depth"], b["depth"])
+    # and the tight trainer works normally afterwards, its buffers enlarged
+    before = tight.repeated_iterations
+    again = tight.run(3)
+    assert tight.repeated_iterations == before and np.isfinite(again)
+    assert np.mean((tight.image() - target) ** 2) * 3 * W * H == pytest.approx(again, rel=1e-3)
+    tight.close()
+    ample.close()
+
+
+def test_a_withheld_update_changes_nothing(gpu, tmp_path):
+    """One iteration from a known state with buffers that are too small, nobody asking for the loss: afterwards the
+    state is that of one complete iteration with step number 3 (not of a step on truncated lists, not of two
+    updates), and the trainer says that it ran one iteration twice."""
+    W = H = 256
+    G = 4000
+    target = trainer.test_pattern(W, H)
+    state = _grown_state(W, H, G, target)
+    path = str(tmp_path / "start.ckpt")
+    t = trainer.Trainer(_config(num_gaussians=G), target)
+    t.run(2)
+    t.set_params(state["params"])
+    t.save_checkpoint(path)
+    t.run(1, want_loss=False)
+    assert t.iteration == 3 and t.repeated_iterations == 1
+    after = t.state()
+    fresh = trainer.Trainer(_config(num_gaussians=G), target)
+    fresh.set_params(state["params"])
+    fresh.run(1)  # waits: sizes its lists for the wide scene
+    fresh.load_checkpoint(path)
+    fresh.run(1)
+    assert fresh.iteration == 3 and fresh.repeated_iterations == 0
+    want = fresh.state()
+    for row in range(9):
+        off = np.abs(after["params"][row] - want["params"][row]) / ROW_LRS[row]
+        assert np.quantile(off, 0.99) <= 0.02 and off.max() <= 2.0, (row, np.quantile(off, 0.99), off.max())
+        g_scale = np.abs(want["m"][row]).max() + 1e-20
+        assert np.abs(after["m"][row] - want["m"][row]).max() <= 1e-3 * g_scale, row
+        v_scale = np.abs(want["v"][row]).max() + 1e-30
+        assert np.abs(after["v"][row] - want["v"][row]).max() <= 1e-3 * v_scale, row
     t.close()
+    fresh.close()
+
+
+def test_a_checkpoint_with_other_depths_loaded_into_a_trainer_that_has_run(gpu, tmp_path):
+    """The renderer keeps the depth order of the depths it saw first (the trainer promises constant depths).  A
+    checkpoint or set_params that brings other depths must make it order again: the continuation equals that of
+    a fresh trainer that loaded the same file."""
+    W, H, G = 96, 64, 500
+    target = trainer.test_pattern(W, H)
+    path = str(tmp_path / "other.ckpt")
+    other = trainer.Trainer(_config(num_gaussians=G, seed=77), target)  # other Gaussians, other depths
+    other.run(5, want_loss=False)
+    other.save_checkpoint(path)
+    used = trainer.Trainer(_config(num_gaussians=G, seed=5), target)
+    used.run(5)  # has ordered by its own depths
+    used.load_checkpoint(path)
+    fresh = trainer.Trainer(_config(num_gaussians=G, seed=5), target)
+    fresh.load_checkpoint(path)
+    la = used.run(1)
+    lb = fresh.run(1)
+    assert abs(la - lb) <= 1e-6 * lb
+    np.testing.assert_array_equal(used.image(), fresh.image())  # same lists, same order: the same image bit for bit
+    used.run(6, want_loss=False)  # iterations that do not report a loss: nothing may have been composited in a stale order
+    fresh.run(6, want_loss=False)
+    la, lb = used.run(1), fresh.run(1)
+    assert abs(la - lb) <= 1e-3 * lb and used.iteration == fresh.iteration == 13
+    # and through set_params
+    s = other.state()
+    used.set_params(depth=s["depth"][::-1].copy())
+    fresh2 = trainer.Trainer(_config(num_gaussians=G, seed=5), target)
+    fresh2.set_params(params=used.state()["params"], depth=s["depth"][::-1].copy())
+    used.run(1)
+    fresh2.run(1)
+    np.testing.assert_array_equal(used.image(), fresh2.image())
+    for t in (other, used, fresh, fresh2):
+        t.close()
 
 
 def test_checkpoint_round_trip_and_resume(gpu, tmp_path, xad):

@@ -48,6 +48,8 @@ SIGNATURES = {
     "xad_host_splat_step_f32": [_int, _int, _int, _vp, _vp, _vp, _vp, _vp, ctypes.POINTER(ctypes.c_double), ctypes.POINTER(_u64), _int],
     "xad_splat_get_stats": [_vp, ctypes.POINTER(_u64), ctypes.POINTER(ctypes.c_uint32), ctypes.POINTER(_flt)],
     "xad_adam_step_f32": [_sz, _int, _vp, _vp, _vp, _vp, ctypes.POINTER(_flt), _flt, _flt, _flt, _int, _vp],
+    "xad_adam_step_gated_f32": [_sz, _int, _vp, _vp, _vp, _vp, ctypes.POINTER(_flt), _flt, _flt, _flt, _int, _vp, _vp, _vp],
+    "xad_splat_overflow_word": [_vp, ctypes.POINTER(_vp)],
     "xad_training_config_defaults": [_vp],
     "xad_training_config_parse": [_int, ctypes.POINTER(ctypes.c_char_p), _vp],
     "xad_training_config_validate": [_vp],
@@ -60,6 +62,7 @@ SIGNATURES = {
     "xad_trainer_destroy": [_vp],
     "xad_trainer_run": [_vp, _int, ctypes.POINTER(ctypes.c_double)],
     "xad_trainer_iteration": [_vp],
+    "xad_trainer_repeated_iterations": [_vp],
     "xad_trainer_download_image": [_vp, _vp],
     "xad_trainer_get_state": [_vp, _vp, _vp, _vp, _vp],
     "xad_trainer_set_params": [_vp, _vp, _vp],
@@ -76,7 +79,8 @@ SIGNATURES = {
     "xad_host_rng_uniform_f32": [_vp, _sz, _u64, _u64, _flt, _flt],
 }
 _RESTYPE = {"xad_last_error": ctypes.c_char_p, "xad_source_digest": ctypes.c_char_p, "xad_training_usage": ctypes.c_char_p,
-            "xad_training_config_defaults": None, "xad_image_free": None, "xad_trainer_destroy": None, "xad_splat_destroy": None}
+            "xad_training_config_defaults": None, "xad_image_free": None, "xad_trainer_destroy": None, "xad_splat_destroy": None,
+            "xad_trainer_repeated_iterations": ctypes.c_longlong}
 
 
 def load():

@@ -377,7 +377,8 @@ __global__ void __launch_bounds__(256) plan_kernel(BinPlan p, const std::uint32_
         // this step's verdict starts here; the last kernel of the binning may still raise it
         const bool overflow = super_pairs > p.capacity_a || carried > p.waves_b;
         status[kStatusOverflow] = overflow ? 1u : 0u;
-        if (overflow) atomicMax(status + kStatusOverflowSticky, super_pairs > p.capacity ? super_pairs : p.capacity + 1);
+        // the sticky word keeps the largest room any step would have needed (never zero for a step that overflowed)
+        if (overflow) atomicMax(status + kStatusOverflowSticky, super_pairs > 0 ? super_pairs : 1u);
         if (clear_depth_flag) status[kStatusDepthChanged] = 0;  // the projection of this step has set it, the host has its copy
     }
 }

@@ -12,6 +12,7 @@ namespace {
 // What the device reports back, in pinned host memory: the status words of the step and the loss.
 struct HostReport {
     std::uint32_t status[kStatusWords];
+    std::uint32_t depth_changed;  // the depth flag as it stood before the binning cleared it
     double loss;
 };
 
@@ -179,16 +180,40 @@ int clear_status(xad_splat_context* c, hipStream_t s, int first, int count) {
     return XAD_OK;
 }
 
+// Room for a scene of `pairs` pairs that keeps growing: half as much again.
 std::uint32_t grown(std::uint32_t pairs) {
-    const std::uint64_t want = static_cast<std::uint64_t>(pairs) + pairs / 4 + 1024;
+    const std::uint64_t want = static_cast<std::uint64_t>(pairs) + pairs / 2 + 1024;
     return static_cast<std::uint32_t>(want < 0xfffffff0ull ? want : 0xfffffff0ull);
+}
+
+// Level A's share of the buffers once a scene's supertile pairs are known: twice that many (the wavefronts
+// launched at level B follow it, so it is not simply everything).
+std::uint32_t level_a_share(std::uint32_t super_pairs) {
+    const std::uint64_t want = 2ull * super_pairs + 1024;
+    return static_cast<std::uint32_t>(want < 0xfffffff0ull ? want : 0xfffffff0ull);
+}
+
+// A step needed room for `seen` pairs (tile or supertile level, whichever is larger) and did not have it.
+// If the buffers themselves are large enough, only level A's share of them was too small: it gets the whole
+// buffer back, nothing is allocated.  Otherwise the buffers are replaced by larger ones.
+int make_room(xad_splat_context* c, std::uint32_t seen) {
+    if (seen <= c->plan.capacity && c->plan.capacity_a < c->plan.capacity) {
+        c->plan = make_bin_plan(c->G, c->tiles_x, c->tiles_y, c->plan.capacity, c->plan.capacity);
+        c->capacity_seen = false;
+        return XAD_OK;
+    }
+    return size_pair_buffers(c, grown(seen > c->plan.capacity ? seen : c->plan.capacity + 1));
+}
+
+std::uint32_t pairs_needed(const HostReport* r) {
+    return r->status[kStatusPairs] > r->status[kStatusSuperPairs] ? r->status[kStatusPairs] : r->status[kStatusSuperPairs];
 }
 
 // Project and bin; leaves the tiles' lists in the context.  Where the host has to look:
 //   - XAD_SPLAT_DEPTH_CHECKED: whether a depth changed, every call (the binning is queued before the
 //     wait and runs during it; if a depth did change, order and binning are redone);
-//   - the first call after the pair lists were sized: whether the pairs fit (if not, the lists are
-//     enlarged and the binning is redone).
+//   - the first call after the pair lists were sized, and every call that waits for the depth flag
+//     anyway: whether the pairs fit (if not, the lists are enlarged and the binning is redone).
 // Otherwise nothing is read back: an overflow or a depth that changed against the caller's promise is
 // left in the sticky status words for the next call that waits anyway.
 int bin(xad_splat_context* c, const float* params, const float* depth, hipStream_t s, bool first_attempt = true) {
@@ -211,36 +236,42 @@ int bin(xad_splat_context* c, const float* params, const float* depth, hipStream
     if (check_depth) {
         // the order of the previous call is used on the assumption that the depths are the same; the
         // flag says whether they were.  The copy is ahead of the binning, which clears the flag.
-        XAD_HIP_TRY(hipMemcpyAsync(c->report->status + kStatusDepthChanged, c->status + kStatusDepthChanged, sizeof(std::uint32_t),
+        XAD_HIP_TRY(hipMemcpyAsync(&c->report->depth_changed, c->status + kStatusDepthChanged, sizeof(std::uint32_t),
                                    hipMemcpyDeviceToHost, s));
-        XAD_HIP_TRY(hipEventRecord(c->report_ready, s));
     }
     // in the static mode the flag stays up until the host has seen it; otherwise every binning clears it
     if (int st = bin_lists(c, s, c->depth_mode != XAD_SPLAT_DEPTH_STATIC)) return st;
-    if (check_depth) {
-        XAD_HIP_TRY(hipEventSynchronize(c->report_ready));
-        if (c->report->status[kStatusDepthChanged] != 0) {
+    if (check_depth || !c->capacity_seen) {
+        // the one wait of this call: the status words of the binning, and with them the depth flag copied above
+        if (int st = fetch_report(c, s)) return st;
+        if (check_depth && c->report->depth_changed != 0) {
             if (int st = order_by_depth(c, depth, s)) return st;
             if (int st = project(false)) return st;  // the rectangles in the new order
             if (int st = bin_lists(c, s, true)) return st;
+            if (int st = fetch_report(c, s)) return st;
         }
-    }
-    if (!c->capacity_seen) {
         // The tile-level pair count is exact even when it exceeds the capacity, unless the supertile lists
         // were cut short as well (then it is a lower bound and the next attempt's count is exact).
-        for (int attempt = 0;; ++attempt) {
-            if (int st = fetch_report(c, s)) return st;
-            if (c->report->status[kStatusOverflow] == 0) break;
-            const std::uint32_t seen = c->pairs > c->report->status[kStatusSuperPairs] ? c->pairs : c->report->status[kStatusSuperPairs];
-            XAD_REQUIRE(attempt < 3 && seen < 0xfffffff0u, "splat: the pair lists overflow at %u pairs", seen);
-            if (int st = size_pair_buffers(c, grown(seen > c->plan.capacity ? seen : c->plan.capacity + 1))) return st;
+        bool made_room = false;
+        for (int attempt = 0; c->report->status[kStatusOverflow] != 0; ++attempt) {
+            const std::uint32_t seen = pairs_needed(c->report);
+            XAD_REQUIRE(attempt < 4 && seen < 0xfffffff0u, "splat: the pair lists overflow at %u pairs", seen);
+            if (int st = make_room(c, seen)) return st;
             if (int st = bin_lists(c, s, false)) return st;
+            if (int st = fetch_report(c, s)) return st;
+            made_room = true;
         }
-        c->capacity_seen = true;
-        // from now on level A is given only the room this scene needs, with a margin: fewer wavefronts at level B
-        // (an overflow of that margin is reported like any other and resets it)
-        c->plan = make_bin_plan(c->G, c->tiles_x, c->tiles_y, c->plan.capacity, grown(c->report->status[kStatusSuperPairs]));
-        if (int st = clear_status(c, s, kStatusOverflowSticky, 1)) return st;
+        if (!c->capacity_seen) {
+            c->capacity_seen = true;
+            // from now on level A is given only the room this scene needs, with a margin: fewer wavefronts at level B
+            // (an overflow of that margin is reported like any other and gives level A the whole buffer back)
+            c->plan = make_bin_plan(c->G, c->tiles_x, c->tiles_y, c->plan.capacity, level_a_share(c->report->status[kStatusSuperPairs]));
+        }
+        // what this call's own attempts left in the sticky word is settled; what earlier calls left there stays
+        if (made_room && c->report->status[kStatusStickyBefore] == 0) {
+            if (int st = clear_status(c, s, kStatusOverflowSticky, 1)) return st;
+            c->report->status[kStatusOverflowSticky] = 0;
+        }
     }
     mark(c, 2, s);
     return XAD_OK;
@@ -267,7 +298,8 @@ int settle_report(xad_splat_context* c, hipStream_t s, const char* who) {
     if (c->report->status[kStatusOverflowSticky] != 0) {
         const std::uint32_t seen = c->report->status[kStatusOverflowSticky];
         (void)clear_status(c, s, kStatusOverflowSticky, 1);
-        if (int grow = size_pair_buffers(c, grown(seen > c->plan.capacity ? seen : c->plan.capacity * 2))) return grow;
+        c->report->status[kStatusOverflowSticky] = 0;
+        if (int grow = make_room(c, seen)) return grow;
         st = xad::fail(XAD_ERR_INCOMPLETE,
                        "%s: a call that did not wait for the device produced more pairs (%u) than the lists held; its image and "
                        "gradients were incomplete.  The lists have been enlarged",
@@ -398,7 +430,7 @@ extern "C" int xad_splat_step(xad_splat_context* c, const float* params, const f
             // this very step did not fit (the scene grew): enlarge the lists and do it again.  Whether steps
             // before it overflowed too is in the word the step saved when it began.
             earlier_steps_overflowed = c->report->status[kStatusStickyBefore] != 0;
-            if (int st = size_pair_buffers(c, grown(c->pairs > c->plan.capacity ? c->pairs : c->plan.capacity * 2))) return st;
+            if (int st = make_room(c, pairs_needed(c->report))) return st;
             if (int st = clear_status(c, s, kStatusOverflowSticky, 1)) return st;
             c->report->status[kStatusOverflowSticky] = 0;
             continue;
@@ -445,6 +477,18 @@ extern "C" int xad_splat_get_stats(xad_splat_context* c, std::uint64_t* pairs, s
     }
     if (stage_ms)
         for (int i = 0; i < xad_splat_context::kStages; ++i) stage_ms[i] = c->stage_ms[i];
+    if (pairs || longest_list) {
+        // this call has waited: what calls that did not wait have left behind is reported (and dealt with) here
+        const int st = settle_report(c, nullptr, who);
+        XAD_HIP_TRY(hipDeviceSynchronize());
+        return st;
+    }
+    return XAD_OK;
+}
+
+extern "C" int xad_splat_overflow_word(xad_splat_context* c, const std::uint32_t** device_word) {
+    XAD_REQUIRE(c && device_word, "xad_splat_overflow_word: null argument");
+    *device_word = c->status + kStatusOverflowSticky;
     return XAD_OK;
 }
 
@@ -455,7 +499,14 @@ extern "C" int xad_splat_get_lists(xad_splat_context* c, std::uint32_t* range_be
     XAD_HIP_TRY(hipDeviceSynchronize());
     XAD_HIP_TRY(hipMemcpy(c->report->status, c->status, sizeof(std::uint32_t) * kStatusWords, hipMemcpyDeviceToHost));
     c->pairs = c->report->status[kStatusPairs];
-    XAD_REQUIRE(c->report->status[kStatusOverflow] == 0, "%s: the last step's lists overflowed", who);
+    {
+        // the lists of a step that outgrew the buffers are not handed out: the buffers are enlarged instead
+        const bool cut_short = c->report->status[kStatusOverflow] != 0;
+        const int st = settle_report(c, nullptr, who);
+        XAD_HIP_TRY(hipDeviceSynchronize());
+        if (st) return st;
+        XAD_REQUIRE(!cut_short, "%s: the last step's lists overflowed", who);
+    }
     XAD_HIP_TRY(hipMemcpy(range_begin, c->range_begin, sizeof(std::uint32_t) * c->tiles, hipMemcpyDeviceToHost));
     XAD_HIP_TRY(hipMemcpy(range_end, c->range_end, sizeof(std::uint32_t) * c->tiles, hipMemcpyDeviceToHost));
     if (gaussians) {

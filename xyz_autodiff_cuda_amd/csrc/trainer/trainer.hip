@@ -17,17 +17,27 @@
 #include "checkpoint.h"
 #include "image_io.h"
 
+// How far the host may run ahead of the device: every kProbeEvery iterations the count of withheld updates is
+// copied to one of kProbeSlots pinned words, and a slot is waited for before it is used again.
+constexpr int kProbeEvery = 8;
+constexpr int kProbeSlots = 4;
+
 struct xad_trainer {
     xad_training_config config;
     int width = 0, height = 0, gaussians = 0;
     int iteration = 0;
+    long long repeated = 0;  // iterations run a second time because their first run did not fit the tile lists
     int device = 0;
     hipStream_t stream = nullptr;
     xad_splat_context* splat = nullptr;
-    // one allocation: params | grads | m | v (9G each) | depth (G)
+    // one allocation: params | grads | m | v (9G each) | depth (G) | the count of withheld updates (one word)
     float* state = nullptr;
     float* target = nullptr;
     float* image = nullptr;
+    const std::uint32_t* overflow_word = nullptr;  // device: not zero while a step's lists have overflowed unseen by the host
+    std::uint32_t* probe = nullptr;                // pinned: kProbeSlots copies of the count + one for the final read
+    hipEvent_t probe_done[kProbeSlots] = {};
+    bool probe_pending[kProbeSlots] = {};
 
     std::size_t g() const { return static_cast<std::size_t>(gaussians); }
     std::size_t pixels() const { return static_cast<std::size_t>(width) * height; }
@@ -36,6 +46,7 @@ struct xad_trainer {
     float* m() const { return state + 18 * g(); }
     float* v() const { return state + 27 * g(); }
     float* depth() const { return state + 36 * g(); }
+    std::uint32_t* withheld() const { return reinterpret_cast<std::uint32_t*>(state + 37 * g()); }
 };
 
 namespace {
@@ -89,10 +100,14 @@ int create(const xad_training_config* config, int width, int height, const float
     if (int st = xad_splat_create(width, height, t->gaussians, 0, &t->splat)) return st;
     // depth is drawn once and never trained: promise that, so that an iteration never waits for the device
     if (int st = xad_splat_set_depth_mode(t->splat, XAD_SPLAT_DEPTH_STATIC)) return st;
-    XAD_HIP_TRY(hipMalloc(&t->state, 37 * t->g() * sizeof(float)));
+    if (int st = xad_splat_overflow_word(t->splat, &t->overflow_word)) return st;
+    XAD_HIP_TRY(hipMalloc(&t->state, (37 * t->g() + 1) * sizeof(float)));
     XAD_HIP_TRY(hipMalloc(&t->target, 3 * t->pixels() * sizeof(float)));
     XAD_HIP_TRY(hipMalloc(&t->image, 3 * t->pixels() * sizeof(float)));
-    XAD_HIP_TRY(hipMemsetAsync(t->state, 0, 37 * t->g() * sizeof(float), t->stream));
+    XAD_HIP_TRY(hipHostMalloc(reinterpret_cast<void**>(&t->probe), (kProbeSlots + 1) * sizeof(std::uint32_t)));
+    for (int k = 0; k <= kProbeSlots; ++k) t->probe[k] = 0;
+    for (auto& e : t->probe_done) XAD_HIP_TRY(hipEventCreateWithFlags(&e, hipEventDisableTiming));
+    XAD_HIP_TRY(hipMemsetAsync(t->state, 0, (37 * t->g() + 1) * sizeof(float), t->stream));
     XAD_HIP_TRY(hipMemsetAsync(t->image, 0, 3 * t->pixels() * sizeof(float), t->stream));
     std::vector<float> params, depth;
     initial_gaussians(*t, params, depth);
@@ -136,10 +151,35 @@ extern "C" void xad_trainer_destroy(xad_trainer* t) {
     if (t->state) (void)hipFree(t->state);
     if (t->target) (void)hipFree(t->target);
     if (t->image) (void)hipFree(t->image);
+    if (t->probe) (void)hipHostFree(t->probe);
+    for (auto& e : t->probe_done)
+        if (e) (void)hipEventDestroy(e);
     if (t->stream) (void)hipStreamDestroy(t->stream);
     delete t;
 }
 
+namespace {
+
+// Waits for the stream and takes the count of updates that were withheld since it was last taken.
+int take_withheld(xad_trainer* t, std::uint32_t* count) {
+    std::uint32_t* slot = t->probe + kProbeSlots;
+    XAD_HIP_TRY(hipMemcpyAsync(slot, t->withheld(), sizeof(std::uint32_t), hipMemcpyDeviceToHost, t->stream));
+    XAD_HIP_TRY(hipMemsetAsync(t->withheld(), 0, sizeof(std::uint32_t), t->stream));
+    XAD_HIP_TRY(hipStreamSynchronize(t->stream));
+    for (bool& pending : t->probe_pending) pending = false;  // whatever the probes would say is in this count
+    *count = *slot;
+    return XAD_OK;
+}
+
+}  // namespace
+
+// An iteration that does not report its loss only queues work, so nobody looks at whether its tile lists
+// fitted their buffers.  The update is therefore gated on the device: xad_adam_step_gated_f32 leaves
+// parameters and moments alone from the first step whose lists overflowed until the host has dealt with it,
+// and counts the updates it withheld.  With the parameters frozen every later iteration repeats the one that
+// overflowed.  Whenever the host next looks (a reported loss, a probe, the end of the run), it takes that
+// count, steps the iteration number back by it, has the lists enlarged by a step that waits, and runs those
+// iterations again: every update that is applied used complete gradients and its own step number.
 extern "C" int xad_trainer_run(xad_trainer* t, int iterations, double* loss_out) {
     XAD_REQUIRE(t, "trainer must not be null");
     XAD_REQUIRE(iterations >= 0, "iterations must not be negative");
@@ -147,30 +187,69 @@ extern "C" int xad_trainer_run(xad_trainer* t, int iterations, double* loss_out)
     const xad_training_config& c = t->config;
     const float learning_rates[9] = {c.lr_center, c.lr_center, c.lr_scale, c.lr_scale, c.lr_rotation,
                                      c.lr_color,  c.lr_color,  c.lr_color, c.lr_opacity};
-    int late = XAD_OK;
-    for (int i = 0; i < iterations; ++i) {
-        double* loss = (i + 1 == iterations) ? loss_out : nullptr;
-        int st = xad_splat_step(t->splat, t->params(), t->depth(), t->target, t->image, t->grads(), loss, t->stream);
-        if (st == XAD_ERR_INCOMPLETE) {
-            // this step is complete (a step that asks for its loss always is); the report is about earlier
-            // iterations, whose updates have been applied: the run goes on and the caller is told at the end
-            late = st;
-            st = XAD_OK;
+    const int target = t->iteration + iterations;
+    bool look = false;  // the next step waits for the device (it follows iterations that have to be run again)
+    double unused = 0.0;
+    int queued = 0;
+    for (;;) {
+        while (t->iteration < target) {
+            const bool last = t->iteration + 1 == target;
+            double* loss = (last && loss_out) ? loss_out : (look ? &unused : nullptr);
+            int st = xad_splat_step(t->splat, t->params(), t->depth(), t->target, t->image, t->grads(), loss, t->stream);
+            // XAD_ERR_INCOMPLETE: this step is complete, steps before it were not; their updates were withheld,
+            // which the count below says more precisely
+            if (st != XAD_OK && st != XAD_ERR_INCOMPLETE) return st;
+            if (loss) {
+                std::uint32_t withheld = 0;
+                if (int st = take_withheld(t, &withheld)) return st;
+                look = false;
+                if (withheld != 0) {
+                    // the parameters are those of `withheld` iterations ago: this step belongs to that iteration
+                    // number.  The lists fit now; go back and run from there (the step just computed is discarded)
+                    t->iteration -= static_cast<int>(withheld);
+                    t->repeated += withheld;
+                    look = true;
+                    continue;
+                }
+            }
+            if (int st = xad_adam_step_gated_f32(t->g(), 9, t->params(), t->grads(), t->m(), t->v(), learning_rates, c.beta1,
+                                                 c.beta2, c.epsilon, t->iteration + 1, t->overflow_word, t->withheld(), t->stream))
+                return st;
+            ++t->iteration;
+            if (++queued % kProbeEvery == 0) {
+                // a look at the count that costs no wait unless the host is kProbeSlots probes ahead of the device:
+                // the probes that have arrived are read, the slot to be used again is waited for
+                const int reuse = (queued / kProbeEvery) % kProbeSlots;
+                bool withholding = false;
+                for (int k = 0; k < kProbeSlots; ++k) {
+                    if (!t->probe_pending[k]) continue;
+                    if (k == reuse) {
+                        XAD_HIP_TRY(hipEventSynchronize(t->probe_done[k]));
+                    } else {
+                        const hipError_t e = hipEventQuery(t->probe_done[k]);
+                        if (e == hipErrorNotReady) continue;
+                        XAD_HIP_TRY(e);
+                    }
+                    t->probe_pending[k] = false;
+                    withholding = withholding || t->probe[k] != 0;
+                }
+                if (withholding) break;  // updates are being withheld: stop queueing, settle below
+                XAD_HIP_TRY(hipMemcpyAsync(t->probe + reuse, t->withheld(), sizeof(std::uint32_t), hipMemcpyDeviceToHost, t->stream));
+                XAD_HIP_TRY(hipEventRecord(t->probe_done[reuse], t->stream));
+                t->probe_pending[reuse] = true;
+            }
         }
-        if (st) return st;
-        if (int st = xad_adam_step_f32(t->g(), 9, t->params(), t->grads(), t->m(), t->v(), learning_rates, c.beta1,
-                                       c.beta2, c.epsilon, t->iteration + 1, t->stream))
-            return st;
-        ++t->iteration;
+        std::uint32_t withheld = 0;
+        if (int st = take_withheld(t, &withheld)) return st;
+        if (withheld == 0 && t->iteration >= target) break;
+        t->iteration -= static_cast<int>(withheld);
+        t->repeated += withheld;
+        look = withheld != 0;
     }
-    XAD_HIP_TRY(hipStreamSynchronize(t->stream));
-    if (late)
-        return xad::fail(late,
-                         "xad_trainer_run: all %d iterations were run, but in some iteration since the last reported loss the "
-                         "tile lists had outgrown their buffers and its gradients lacked contributions; the buffers have been enlarged",
-                         iterations);
     return XAD_OK;
 }
+
+extern "C" long long xad_trainer_repeated_iterations(const xad_trainer* t) { return t ? t->repeated : -1; }
 
 extern "C" int xad_trainer_iteration(const xad_trainer* t) { return t ? t->iteration : -1; }
 
@@ -199,8 +278,11 @@ extern "C" int xad_trainer_set_params(xad_trainer* t, const float* params, const
     if (int st = bind_device(t)) return st;
     if (params)
         if (int st = upload(t, t->params(), params, 9 * t->g())) return st;
-    if (depth)
+    if (depth) {
         if (int st = upload(t, t->depth(), depth, t->g())) return st;
+        // the renderer keeps the order of the depths it saw first (static mode): it has to order again
+        if (int st = xad_splat_set_depth_mode(t->splat, XAD_SPLAT_DEPTH_STATIC)) return st;
+    }
     return XAD_OK;
 }
 
@@ -249,6 +331,7 @@ extern "C" int xad_trainer_load_checkpoint(xad_trainer* t, const char* path) {
     if (int st = upload(t, t->m(), state.m.data(), state.m.size())) return st;
     if (int st = upload(t, t->v(), state.v.data(), state.v.size())) return st;
     if (int st = upload(t, t->depth(), state.depth.data(), state.depth.size())) return st;
+    if (int st = xad_splat_set_depth_mode(t->splat, XAD_SPLAT_DEPTH_STATIC)) return st;  // other depths: order again
     t->iteration = h.iteration;
     return XAD_OK;
 }

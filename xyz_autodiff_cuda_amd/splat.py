@@ -6,6 +6,7 @@ xyz-autodiff-cuda): zero/compute gradients, read the loss, Adam step.
 """
 import ctypes
 import math
+import warnings
 
 from . import _lib, rng
 
@@ -75,6 +76,12 @@ class SplatContext:
         _lib.check(st, "xad_splat_get_lists")
         return begin, end, ids[:pairs]
 
+    def overflow_word(self):
+        """Device address of the word that is not zero while a step's lists have overflowed unseen by the host."""
+        word = ctypes.c_void_p()
+        _lib.check(self._lib.xad_splat_overflow_word(self._handle, ctypes.byref(word)), "xad_splat_overflow_word")
+        return word.value
+
     def set_profiling(self, enabled):
         _lib.check(self._lib.xad_splat_set_profiling(self._handle, 1 if enabled else 0), "xad_splat_set_profiling")
 
@@ -110,7 +117,11 @@ class SplatContext:
         with torch.cuda.device(self.device):
             st = self._lib.xad_splat_step(self._handle, params.data_ptr(), depth.data_ptr(), target.data_ptr(), image.data_ptr(),
                                           grads.data_ptr(), ctypes.byref(loss) if want_loss else None, self._stream(stream))
-        _lib.check(st, "xad_splat_step")
+        if st == _lib.XAD_ERR_INCOMPLETE:
+            # this step's outputs are complete; an earlier step that did not wait lacked pairs (lists since enlarged)
+            warnings.warn(self._lib.xad_last_error().decode("utf-8", "replace"), RuntimeWarning)
+        else:
+            _lib.check(st, "xad_splat_step")
         return image, grads, (loss.value if want_loss else None)
 
     def stats(self, longest_list=False):
@@ -150,8 +161,12 @@ def host_step(params, depth, target, width, height, want_grads=True, num_threads
     return {"image": image, "grads": grads, "loss": loss.value, "pairs": pairs.value}
 
 
-def adam_step(params, grads, m, v, learning_rates, iteration, beta1=0.9, beta2=0.999, eps=1e-8, stream=None):
-    """In-place Adam over (rows, n) tensors; learning_rates: one float per row (or one float for all)."""
+def adam_step(params, grads, m, v, learning_rates, iteration, beta1=0.9, beta2=0.999, eps=1e-8, stream=None,
+              hold_if_nonzero=None, held_count=None):
+    """In-place Adam over (rows, n) tensors; learning_rates: one float per row (or one float for all).
+    hold_if_nonzero (a device address, e.g. SplatContext.overflow_word(), or a one-element int32 CUDA tensor): the
+    update is decided on the device and withheld when that word is not zero; held_count (one-element int32 CUDA
+    tensor) then counts it."""
     import torch
 
     rows, n = params.shape
@@ -164,8 +179,14 @@ def adam_step(params, grads, m, v, learning_rates, iteration, beta1=0.9, beta2=0
     lrs = (ctypes.c_float * rows)(*[float(x) for x in learning_rates])
     s = (stream if stream is not None else torch.cuda.current_stream(params.device)).cuda_stream
     with torch.cuda.device(params.device):
-        st = _lib.load().xad_adam_step_f32(n, rows, params.data_ptr(), grads.data_ptr(), m.data_ptr(), v.data_ptr(), lrs,
-                                           beta1, beta2, eps, int(iteration), s)
+        if hold_if_nonzero is None:
+            st = _lib.load().xad_adam_step_f32(n, rows, params.data_ptr(), grads.data_ptr(), m.data_ptr(), v.data_ptr(), lrs,
+                                               beta1, beta2, eps, int(iteration), s)
+        else:
+            gate = hold_if_nonzero.data_ptr() if hasattr(hold_if_nonzero, "data_ptr") else int(hold_if_nonzero)
+            st = _lib.load().xad_adam_step_gated_f32(n, rows, params.data_ptr(), grads.data_ptr(), m.data_ptr(), v.data_ptr(), lrs,
+                                                     beta1, beta2, eps, int(iteration), gate,
+                                                     held_count.data_ptr() if held_count is not None else None, s)
     _lib.check(st, "xad_adam_step_f32")
 
 

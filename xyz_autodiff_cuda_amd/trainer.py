@@ -6,7 +6,6 @@ training_config.cpp, image_utils.cpp} in xyz-autodiff-cuda.  The command-line
 program built next to the library, xad_splat_train, uses the same entry points.
 """
 import ctypes
-import warnings
 import os
 
 import numpy as np
@@ -119,12 +118,13 @@ class Trainer:
     def run(self, iterations, want_loss=True):
         loss = ctypes.c_double(0.0)
         status = self._lib.xad_trainer_run(self._handle, int(iterations), ctypes.byref(loss) if want_loss else None)
-        if status == _lib.XAD_ERR_INCOMPLETE:
-            # every iteration has run; some earlier one lacked contributions (buffers outgrown, since enlarged)
-            warnings.warn(self._lib.xad_last_error().decode("utf-8", "replace"), RuntimeWarning)
-        else:
-            _lib.check(status, "xad_trainer_run")
+        _lib.check(status, "xad_trainer_run")
         return loss.value if want_loss else None
+
+    @property
+    def repeated_iterations(self):
+        """Iterations run a second time because their tile lists had outgrown the buffers (their first run changed nothing)."""
+        return self._lib.xad_trainer_repeated_iterations(self._handle)
 
     @property
     def iteration(self):
