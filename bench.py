@@ -27,6 +27,14 @@ TRAFFIC_SOURCE = {"profile": "profiles/chain_single_kernel_hbm_traffic.md", "byt
                   "note": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of `bench.py --counter-probe chain`, each scaled by a copy of "
                           "known size; a constant from that profile, not a reading of this run"}
 N_FULL = 64 * 1024 * 1024
+# Atomic requests that reach L2 in one iteration of the splatting step, from counter passes over
+# `bench.py --counter-probe splat` / `--counter-probe splat4` (TCC_ATOMIC_sum per kernel, summed over the
+# iteration's kernels); constants from those profiles, not readings of this run.
+ATOMIC_TRAFFIC = {
+    "config5_200k_2048": {"l2_atomic_requests_measured": 3_665_995, "pairs_in_that_run": 5_484_589,
+                          "values_added": 39_000_000,
+                          "source": "profiles/splat_200k_2048_kernel_counters.md (TCC_ATOMIC_sum: render_backward_kernel 3 665 877, scans 118)"},
+}
 
 
 def cpu_baseline(host_inputs, budget_s=12.0):
@@ -158,11 +166,22 @@ def trainer_report():
     config = trainer.TrainingConfig.defaults(num_gaussians=G, seed=1, target_image_path="synthetic")
     t = trainer.Trainer(config, target)
     first = t.run(5)
+    repeated_before = t.repeated_iterations
     t0 = time.perf_counter()
     last = t.run(50)
     dt = time.perf_counter() - t0
+    repeated = t.repeated_iterations - repeated_before
+    # a second stretch, for a figure without the repeats of the first (the lists have been enlarged by then)
+    t0 = time.perf_counter()
+    t.run(50, want_loss=False)
+    dt2 = time.perf_counter() - t0
+    repeated2 = t.repeated_iterations - repeated_before - repeated
     t.close()
+    # ms_per_iter divides by the 50 iterations that count; the timed region also ran `repeated_iterations` of them twice
+    # (their first run found the tile lists too small and changed nothing: the update is withheld on the device)
     return {"gaussians": G, "image": [W, H], "iterations": 50, "iters_per_s": 50 / dt, "ms_per_iter": dt / 50 * 1e3,
+            "repeated_iterations": int(repeated), "ms_per_iteration_run": dt / (50 + repeated) * 1e3,
+            "next_50": {"ms_per_iter": dt2 / 50 * 1e3, "repeated_iterations": int(repeated2)},
             "loss_after_5": first, "loss_after_55": last}
 
 
@@ -238,20 +257,33 @@ def splat_report(with_oracle, iters=30):
         m, v = torch.zeros_like(params), torch.zeros_like(params)
         image = torch.empty(H, W, 3, device=dev)
         grads = torch.empty(9, G, device=dev)
+        # no update on gradients from lists that have outgrown their buffers: decided on the device, counted here
+        gate, held = ctx.overflow_word(), torch.zeros(1, dtype=torch.int32, device=dev)
         _, _, first_loss = ctx.step(params, depth, target, image, grads)
         first_grads = grads.cpu().numpy().astype(np.float64) if with_oracle else None
         first_image = image.cpu().numpy() if with_oracle else None
         first_pairs = ctx.stats()["pairs"]
         for it in range(1, 4):
             ctx.step(params, depth, target, image, grads, want_loss=False)
-            splat.adam_step(params, grads, m, v, 1e-2, it)
+            splat.adam_step(params, grads, m, v, 1e-2, it, hold_if_nonzero=gate, held_count=held)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         for it in range(4, 4 + iters):
             ctx.step(params, depth, target, image, grads, want_loss=False)
-            splat.adam_step(params, grads, m, v, 1e-2, it)
+            splat.adam_step(params, grads, m, v, 1e-2, it, hold_if_nonzero=gate, held_count=held)
         torch.cuda.synchronize()
         per_iter = (time.perf_counter() - t0) / iters
+        # the same iterations with the depth order recomputed by every step (what a caller whose depths change pays)
+        ctx.set_depth_mode("every_step")
+        ctx.step(params, depth, target, image, grads, want_loss=False)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for it in range(4 + iters, 4 + 2 * iters):
+            ctx.step(params, depth, target, image, grads, want_loss=False)
+            splat.adam_step(params, grads, m, v, 1e-2, it, hold_if_nonzero=gate, held_count=held)
+        torch.cuda.synchronize()
+        per_iter_every_step = (time.perf_counter() - t0) / iters
+        withheld_updates = int(held)
         a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         a.record()
         for it in range(10):
@@ -259,23 +291,28 @@ def splat_report(with_oracle, iters=30):
         b.record()
         torch.cuda.synchronize()
         adam_ms = a.elapsed_time(b) / 10
-        ctx.set_profiling(True)
+        ctx.set_profiling(True)  # (still in the every_step mode: the split has its sort stage)
         acc = None
         for _ in range(5):
             ctx.step(params, depth, target, image, grads, want_loss=False)
             ms = ctx.stats()["stage_ms"]
             acc = ms if acc is None else {k: acc[k] + ms[k] for k in ms}
         ctx.set_profiling(False)
+        ctx.set_depth_mode("static")
         _, _, last_loss = ctx.step(params, depth, target, image, grads)
         stats = ctx.stats(longest_list=True)
         tiles = ((W + 15) // 16) * ((H + 15) // 16)
         entry = {
             "gaussians": G, "image": [W, H], "iters_per_s": 1.0 / per_iter, "ms_per_iter": per_iter * 1e3,
+            "iters_per_s_every_step": 1.0 / per_iter_every_step, "ms_per_iter_every_step": per_iter_every_step * 1e3,
+            "every_step_over_static": per_iter_every_step / per_iter,
+            "updates_withheld_in_timed_loops": withheld_updates,
             "stage_ms": {**{k: v / 5 for k, v in acc.items()}, "adam": adam_ms},
             "pairs": stats["pairs"], "mean_list": stats["pairs"] / tiles, "longest_list": stats["longest_list"],
-            "global_atomics_per_iter": {"after_block_pre_reduction": stats["pairs"] * 9 + tiles,
-                                        "per_pixel_pair_naive": int(stats["pairs"]) * 256 * 9},
-            "loss_first": first_loss, "loss_after_%d_iters" % (iters + 8): last_loss,
+            "global_atomics_per_iter": {**ATOMIC_TRAFFIC.get(name, {}),
+                                        "values_added_if_one_atomic_per_pair_and_field": stats["pairs"] * 9 + tiles,
+                                        "values_added_if_one_atomic_per_pixel_pair_and_field": int(stats["pairs"]) * 256 * 9},
+            "loss_first": first_loss, "loss_after_%d_iters" % (2 * iters + 10): last_loss,
         }
         if with_oracle:
             from tests import _oracle
@@ -450,6 +487,31 @@ def main():
             policy_ms[name].append(a.elapsed_time(b) / 10)
     store_policy = {name: algorithmic_bytes / (sorted(v)[1] / 1e3) / 1e9 for name, v in policy_ms.items()}
 
+    # what this memory system gives a plain copy in the same process on the same day: one stream in, one out,
+    # 1 GiB each way (far beyond the caches), the median of three rounds of ten launches
+    copy_src = torch.cat(ins[:4]) if n * 4 <= (1 << 28) else torch.cat([t[: (1 << 26)] for t in ins[:4]])
+    copy_dst = torch.empty_like(copy_src)
+    copy_rates = {}
+    for variant in ("chain_pattern_4B_x1_non_temporal",) + instruments.COPY_VARIANTS:
+        def launch():
+            if variant.startswith("chain_pattern"):
+                instruments.stream_copy(copy_src, copy_dst)
+            else:
+                instruments.copy_variant(copy_src, copy_dst, variant)
+        ms = []
+        for _ in range(3):
+            launch()
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            for _ in range(10):
+                launch()
+            b.record()
+            torch.cuda.synchronize()
+            ms.append(a.elapsed_time(b) / 10)
+        copy_rates[variant] = 2.0 * copy_src.numel() * 4 / (sorted(ms)[1] / 1e3) / 1e9
+    copy_ceiling = max(copy_rates.values())
+    del copy_src, copy_dst
+
     record = {
         "metric": "per-thread fwd+bwd evals/sec",
         "value": n * args.steps / wall,
@@ -474,6 +536,9 @@ def main():
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBPS,
+            "copy_ceiling_GBps": copy_ceiling,
+            "copy_GBps_by_shape": copy_rates,
+            "frac_of_copy_ceiling": achieved / copy_ceiling,
             "traffic": MEASURED_TRAFFIC_BYTES_PER_EVAL * n,
             "traffic_source": TRAFFIC_SOURCE,
             "kernel": "chain_single_kernel",

@@ -216,13 +216,15 @@ int xad_splat_step(xad_splat_context* ctx, const float* params, const float* dep
 #define XAD_SPLAT_DEPTH_STATIC 1
 #define XAD_SPLAT_DEPTH_EVERY_STEP 2
 int xad_splat_set_depth_mode(xad_splat_context* ctx, int mode);
-/* Per-stage GPU times (events around project, binning, render forward, render
- * backward, parameter backward) are recorded by the next calls when enabled;
- * recording makes each call wait for the stream. */
+/* Per-stage GPU times (events around depth order, project, binning, render
+ * forward, render backward, parameter backward) are recorded by the next calls
+ * when enabled; recording makes each call wait for the stream. */
 int xad_splat_set_profiling(xad_splat_context* ctx, int enabled);
 /* Of the last call: number of (tile, Gaussian) pairs, longest tile list (either
- * makes the call wait for the device), and the five stage times in milliseconds
- * (zeros unless profiling is enabled).  Any output pointer may be NULL. */
+ * makes the call wait for the device, and reports what calls that did not wait
+ * have left behind, see above), and the six stage times in milliseconds (zeros
+ * unless profiling is enabled; the first is the depth order, close to zero in a
+ * call that kept the order it had).  Any output pointer may be NULL. */
 int xad_splat_get_stats(xad_splat_context* ctx, uint64_t* pairs, uint32_t* longest_list, float* stage_ms);
 /* The tile lists of the last call, to host memory: tile t (row-major) holds
  * gaussians[range_begin[t] .. range_end[t]), in compositing order.  range_begin and
@@ -237,6 +239,15 @@ int xad_splat_get_lists(xad_splat_context* ctx, uint32_t* range_begin, uint32_t*
  * that step's gradients (xad_adam_step_gated_f32).  Valid for the context's life.
  * No counterpart in the reference, whose one kernel needs no lists. */
 int xad_splat_overflow_word(xad_splat_context* ctx, const uint32_t** device_word);
+/* The order in which the step composites: order[i] (device, n words) = the i-th
+ * Gaussian by (depth, index), rank (device, n words) its inverse.  A stable radix
+ * sort on the device (csrc/splat_sort.hip), the one xad_splat_step runs whenever
+ * it has to order (every call in XAD_SPLAT_DEPTH_EVERY_STEP mode).  -0.0 and +0.0
+ * are one depth; a NaN sorts by its bit pattern (first with the sign bit set, last
+ * without).  n < 2^30.  Allocates its workspace and waits for the stream.
+ * No counterpart in the reference, which composites in index order
+ * (gaussian_splatting_kernel.cu:33-62). */
+int xad_depth_order_f32(size_t n, const float* depth, uint32_t* order, uint32_t* rank, void* stream);
 /* The same step on the host cores, every pointer host memory: the CPU figure the
  * GPU step is reported beside.  Tiles are dealt to num_threads threads (0: one per
  * hardware thread); every (pixel, Gaussian) pair builds the renderer's per-pair

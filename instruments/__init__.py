@@ -16,6 +16,7 @@ SIGNATURES = {
     "xadi_chain_forward_backward_f32_layout": [_sz] + [_vp] * 13 + [_int, _vp],
     "xadi_chain_store_policy": [_int, _sz] + [_vp] * 13 + [_vp],
     "xadi_stream_copy_f32": [_sz, _vp, _vp, _vp],
+    "xadi_copy_variant_f32": [_int, _sz, _vp, _vp, _vp],
     "xadi_chain_kernel_resources": [_vp],
     "xadi_lds_atomic_cycles": [_int, _int, ctypes.POINTER(ctypes.c_double)],
 }
@@ -106,6 +107,23 @@ def stream_copy(src, dst, stream=None):
     s = stream if stream is not None else torch.cuda.current_stream(src.device)
     with torch.cuda.device(src.device):
         _check(load().xadi_stream_copy_f32(src.numel(), src.data_ptr(), dst.data_ptr(), s.cuda_stream), "xadi_stream_copy_f32")
+    return dst
+
+
+COPY_VARIANTS = ("4B_x1_write_through", "4B_x8_write_through", "16B_x1_plain", "16B_x4_plain", "16B_x4_non_temporal",
+                 "16B_read_4B_write_through_x2", "4B_x8_plain")
+
+
+def copy_variant(src, dst, variant, stream=None):
+    """dst = src by one of COPY_VARIANTS (name or index)."""
+    import torch
+
+    assert src.is_cuda and dst.is_cuda and src.dtype == dst.dtype == torch.float32 and src.numel() == dst.numel()
+    if isinstance(variant, str):
+        variant = COPY_VARIANTS.index(variant)
+    s = stream if stream is not None else torch.cuda.current_stream(src.device)
+    with torch.cuda.device(src.device):
+        _check(load().xadi_copy_variant_f32(int(variant), src.numel(), src.data_ptr(), dst.data_ptr(), s.cuda_stream), "xadi_copy_variant_f32")
     return dst
 
 

@@ -99,6 +99,32 @@ XADI_EXPORT int xadi_stream_copy_f32(std::size_t n, const float* src, float* dst
     return 0;
 }
 
+XADI_EXPORT int xadi_copy_variant_f32(int variant, std::size_t n, const float* src, float* dst, void* stream) {
+    const char* who = "xadi_copy_variant_f32";
+    if (n == 0) return 0;
+    XAD_REQUIRE(src && dst, "%s: null array", who);
+    XAD_REQUIRE(n % 4 == 0 && xad::aligned16(src) && xad::aligned16(dst), "%s: n must be a multiple of 4 and the arrays 16-byte aligned", who);
+    XAD_REQUIRE(n <= 0x7fffffffull * 64, "%s: n = %zu exceeds the grid limit", who, n);
+    hipStream_t s = xad::as_stream(stream);
+    auto launch = [&](auto kernel, int floats, int in_flight) {
+        const std::size_t per_block = static_cast<std::size_t>(kSingleBlock) * floats * in_flight;
+        hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>((n + per_block - 1) / per_block)), dim3(kSingleBlock), 0, s, src, dst, n);
+    };
+    using xad_chain::copy_variant_kernel;
+    switch (variant) {
+        case 0: launch(copy_variant_kernel<1, 1, StorePolicy::WriteThrough>, 1, 1); break;
+        case 1: launch(copy_variant_kernel<1, 8, StorePolicy::WriteThrough>, 1, 8); break;
+        case 2: launch(copy_variant_kernel<4, 1, StorePolicy::Plain>, 4, 1); break;
+        case 3: launch(copy_variant_kernel<4, 4, StorePolicy::Plain>, 4, 4); break;
+        case 4: launch(copy_variant_kernel<4, 4, StorePolicy::NonTemporal>, 4, 4); break;
+        case 5: launch(copy_variant_kernel<4, 2, StorePolicy::WriteThrough>, 4, 2); break;
+        case 6: launch(copy_variant_kernel<1, 8, StorePolicy::Plain>, 1, 8); break;
+        default: return xad::fail(XAD_ERR_INVALID_ARGUMENT, "%s: variant must be 0..6, got %d", who, variant);
+    }
+    XAD_HIP_TRY(hipGetLastError());
+    return 0;
+}
+
 XADI_EXPORT int xadi_chain_kernel_resources(int* out) {
     XAD_REQUIRE(out, "xadi_chain_kernel_resources: out is null");
     const void* kernel = reinterpret_cast<const void*>(xad_chain::chain_single_kernel<StorePolicy::WriteThrough>);

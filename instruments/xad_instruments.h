@@ -49,6 +49,14 @@ int xadi_chain_store_policy(int policy, size_t n,
  * to calibrate counters and bandwidth against. */
 int xadi_stream_copy_f32(size_t n, const float* src, float* dst, void* stream);
 
+/* The same copy in other shapes, to find the best this memory system gives one stream in and one out:
+ * variant 0: 4 bytes per access, one access per lane, write-through stores; 1: 4 bytes, eight accesses of a
+ * lane in flight, write-through; 2: 16 bytes, one, plain stores; 3: 16 bytes, four in flight, plain;
+ * 4: 16 bytes, four, non-temporal stores; 5: 16 bytes read, written through as four 4-byte stores, two in
+ * flight; 6: 4 bytes, eight in flight, plain.  All loads non-temporal.  n a multiple of 4, arrays 16-byte
+ * aligned. */
+int xadi_copy_variant_f32(int variant, size_t n, const float* src, float* dst, void* stream);
+
 /* Resources of the chain kernel (write-through stores) as the loaded code object and the current
  * device report them: vector registers per lane, scratch (spill) bytes per lane, static LDS bytes per
  * block, lanes per block, and how many such blocks one compute unit holds at once.  out[5], host. */

@@ -50,6 +50,7 @@ SIGNATURES = {
     "xad_adam_step_f32": [_sz, _int, _vp, _vp, _vp, _vp, ctypes.POINTER(_flt), _flt, _flt, _flt, _int, _vp],
     "xad_adam_step_gated_f32": [_sz, _int, _vp, _vp, _vp, _vp, ctypes.POINTER(_flt), _flt, _flt, _flt, _int, _vp, _vp, _vp],
     "xad_splat_overflow_word": [_vp, ctypes.POINTER(_vp)],
+    "xad_depth_order_f32": [_sz, _vp, _vp, _vp, _vp],
     "xad_training_config_defaults": [_vp],
     "xad_training_config_parse": [_int, ctypes.POINTER(ctypes.c_char_p), _vp],
     "xad_training_config_validate": [_vp],

@@ -10,6 +10,7 @@
 // mapping and the plain copy exist so that those choices can be measured again
 // (they are instantiated by the measurement library, not by the product).
 #include <cstddef>
+#include <type_traits>
 
 #include <hip/hip_runtime.h>
 
@@ -94,6 +95,45 @@ __global__ void __launch_bounds__(kSingleBlock) stream_copy_kernel(const float* 
                                                                    std::size_t n) {
     const std::size_t i = static_cast<std::size_t>(blockIdx.x) * kSingleBlock + threadIdx.x;
     if (i < n) __builtin_nontemporal_store(__builtin_nontemporal_load(src + i), dst + i);
+}
+
+// Plain copies in other shapes, to find what this memory system gives a copy at best: kFloats floats per
+// access (1 or 4: 4 or 16 bytes), kInFlight accesses of a lane issued before the first store (each a block's
+// width apart, so every wavefront instruction stays contiguous), stores by policy P.
+template <int kFloats, int kInFlight, StorePolicy P>
+__global__ void __launch_bounds__(kSingleBlock) copy_variant_kernel(const float* __restrict__ src, float* __restrict__ dst,
+                                                                    std::size_t n) {
+    typedef float NativeFloat4 __attribute__((ext_vector_type(4)));
+    using Word = std::conditional_t<kFloats == 4, NativeFloat4, float>;
+    const std::size_t words = n / kFloats;
+    const std::size_t base = static_cast<std::size_t>(blockIdx.x) * kSingleBlock * kInFlight + threadIdx.x;
+    const Word* in = reinterpret_cast<const Word*>(src);
+    Word* out = reinterpret_cast<Word*>(dst);
+    Word v[kInFlight];
+#pragma unroll
+    for (int k = 0; k < kInFlight; ++k) {
+        const std::size_t i = base + static_cast<std::size_t>(k) * kSingleBlock;
+        if (i < words) v[k] = __builtin_nontemporal_load(in + i);
+    }
+#pragma unroll
+    for (int k = 0; k < kInFlight; ++k) {
+        const std::size_t i = base + static_cast<std::size_t>(k) * kSingleBlock;
+        if (i < words) {
+            if constexpr (kFloats == 1) {
+                store_result<P>(out + i, v[k]);
+            } else if constexpr (P == StorePolicy::NonTemporal) {
+                __builtin_nontemporal_store(v[k], out + i);
+            } else if constexpr (P == StorePolicy::WriteThrough) {
+                float* o = reinterpret_cast<float*>(out + i);
+                store_result<P>(o, v[k].x);
+                store_result<P>(o + 1, v[k].y);
+                store_result<P>(o + 2, v[k].z);
+                store_result<P>(o + 3, v[k].w);
+            } else {
+                out[i] = v[k];
+            }
+        }
+    }
 }
 
 }  // namespace xad_chain

@@ -61,7 +61,7 @@ struct xad_splat_context {
 
     HostReport* report = nullptr;  // pinned
 
-    static constexpr int kStages = 5;  // project, binning, render forward, render backward, parameter backward
+    static constexpr int kStages = 6;  // depth order, project, binning, render forward, render backward, parameter backward
     hipEvent_t marks[kStages + 1] = {};
     float stage_ms[kStages] = {};
     hipEvent_t report_ready = nullptr;
@@ -146,16 +146,21 @@ void mark(xad_splat_context* c, int index, hipStream_t s) {
     if (c->profile) (void)hipEventRecord(c->marks[index], s);
 }
 
-// (depth, index) order of the Gaussians, kept until a depth changes
-int order_by_depth(xad_splat_context* c, const float* depth, hipStream_t s) {
-    c->order_valid = false;
-    if (int st = launch_depth_keys(s, c->G, depth, c->depth_keys, c->identity)) return st;
-    if (int st = sort_by_depth(s, c->depth_sort_temp, c->depth_sort_bytes, c->depth_keys, c->depth_keys_sorted, c->identity,
-                               c->by_depth, c->G))
+// Projection, after ordering the Gaussians by (depth, index) when asked to; the order is then kept until a depth changes.
+int project_gaussians(xad_splat_context* c, const float* params, const float* depth, hipStream_t s, bool first_of_step,
+                      bool ordering) {
+    if (ordering) {
+        c->order_valid = false;
+        if (int st = sort_by_depth(s, c->depth_sort_temp, c->depth_sort_bytes, depth, c->depth_keys, c->depth_keys_sorted, c->identity,
+                                   c->by_depth, c->rank, c->ordered_depth, c->G))
+            return st;
+        c->order_valid = true;
+    }
+    mark(c, 1, s);
+    if (int st = launch_project(s, c->G, params, depth, c->ordered_depth, c->rank, c->status, c->width, c->height, c->records,
+                                c->rects, c->rects_by_depth, c->record_grads, c->loss, first_of_step))
         return st;
-    if (int st = launch_depth_rank(s, c->G, c->by_depth, c->rank)) return st;
-    XAD_HIP_TRY(hipMemcpyAsync(c->ordered_depth, depth, sizeof(float) * c->G, hipMemcpyDeviceToDevice, s));
-    c->order_valid = true;
+    mark(c, 2, s);
     return XAD_OK;
 }
 
@@ -224,14 +229,7 @@ int bin(xad_splat_context* c, const float* params, const float* depth, hipStream
         if (int st = size_pair_buffers(c, static_cast<std::uint32_t>(static_cast<std::size_t>(c->G) * 8 + 1024))) return st;
     mark(c, 0, s);
     const bool had_order = c->order_valid && c->depth_mode != XAD_SPLAT_DEPTH_EVERY_STEP;
-    if (!had_order)
-        if (int st = order_by_depth(c, depth, s)) return st;
-    auto project = [&](bool first_of_step) {
-        return launch_project(s, c->G, params, depth, c->ordered_depth, c->rank, c->status, c->width, c->height, c->records,
-                              c->rects, c->rects_by_depth, c->record_grads, c->loss, first_of_step);
-    };
-    if (int st = project(first_attempt)) return st;
-    mark(c, 1, s);
+    if (int st = project_gaussians(c, params, depth, s, first_attempt, !had_order)) return st;
     const bool check_depth = c->depth_mode == XAD_SPLAT_DEPTH_CHECKED && had_order;
     if (check_depth) {
         // the order of the previous call is used on the assumption that the depths are the same; the
@@ -245,8 +243,7 @@ int bin(xad_splat_context* c, const float* params, const float* depth, hipStream
         // the one wait of this call: the status words of the binning, and with them the depth flag copied above
         if (int st = fetch_report(c, s)) return st;
         if (check_depth && c->report->depth_changed != 0) {
-            if (int st = order_by_depth(c, depth, s)) return st;
-            if (int st = project(false)) return st;  // the rectangles in the new order
+            if (int st = project_gaussians(c, params, depth, s, false, true)) return st;  // the new order, the rectangles in it
             if (int st = bin_lists(c, s, true)) return st;
             if (int st = fetch_report(c, s)) return st;
         }
@@ -273,7 +270,7 @@ int bin(xad_splat_context* c, const float* params, const float* depth, hipStream
             c->report->status[kStatusOverflowSticky] = 0;
         }
     }
-    mark(c, 2, s);
+    mark(c, 3, s);
     return XAD_OK;
 }
 
@@ -399,8 +396,8 @@ extern "C" int xad_splat_forward(xad_splat_context* c, const float* params, cons
     if (int st = launch_render_forward(s, c->width, c->height, c->range_begin, c->range_end, c->list, c->records, image,
                                        c->final_T, c->n_contrib, c->segments, c->segment_state, c->tile_order))
         return st;
-    mark(c, 3, s);
-    collect_times(c, 3);
+    mark(c, 4, s);
+    collect_times(c, 4);
     return XAD_OK;
 }
 
@@ -415,14 +412,14 @@ extern "C" int xad_splat_step(xad_splat_context* c, const float* params, const f
         if (int st = launch_render_forward(s, c->width, c->height, c->range_begin, c->range_end, c->list, c->records, image,
                                            c->final_T, c->n_contrib, c->segments, c->segment_state, c->tile_order))
             return st;
-        mark(c, 3, s);
+        mark(c, 4, s);
         if (int st = launch_render_backward(s, c->width, c->height, c->range_begin, c->range_end, c->list, c->records, image,
                                             target, c->final_T, c->n_contrib, c->record_grads, c->loss, c->segments,
                                             c->segment_state, c->tile_order))
             return st;
-        mark(c, 4, s);
-        if (int st = launch_gaussian_backward(s, c->G, params, c->record_grads, grads, c->loss)) return st;
         mark(c, 5, s);
+        if (int st = launch_gaussian_backward(s, c->G, params, c->record_grads, grads, c->loss)) return st;
+        mark(c, 6, s);
         if (!loss_out) break;
         // the loss is read back, and with it what the device has to report
         if (int st = fetch_report(c, s)) return st;
@@ -437,12 +434,12 @@ extern "C" int xad_splat_step(xad_splat_context* c, const float* params, const f
         }
         *loss_out = c->report->loss;
         if (int st = settle_report(c, s, who)) {
-            collect_times(c, 5);
+            collect_times(c, 6);
             return st;
         }
         break;
     }
-    collect_times(c, 5);
+    collect_times(c, 6);
     if (earlier_steps_overflowed)
         return xad::fail(XAD_ERR_INCOMPLETE,
                          "%s: a call that did not wait for the device produced more pairs than the lists held; its image and "

@@ -98,30 +98,6 @@ __global__ void __launch_bounds__(256) project_kernel(int G, const float* __rest
     rects_by_depth[rank[g]] = rc;  // the binning walks the Gaussians in depth order
 }
 
-// Order-preserving map from float to unsigned (any sign).
-__device__ __forceinline__ std::uint32_t ordered_bits(float f) {
-    const std::uint32_t u = __builtin_bit_cast(std::uint32_t, f);
-    return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
-}
-
-__global__ void __launch_bounds__(256) depth_rank_kernel(int G, const std::uint32_t* __restrict__ by_depth,
-                                                         std::uint32_t* __restrict__ rank) {
-    const int i = blockIdx.x * 256 + threadIdx.x;
-    if (i < G) rank[by_depth[i]] = static_cast<std::uint32_t>(i);
-}
-
-// Depth order.  depth_key_kernel writes the order-preserving bits of every depth
-// and the identity permutation; a stable sort of those pairs gives by_depth, the
-// Gaussians in (depth, index) order.  The binning walks the Gaussians in that
-// order, which leaves every tile's list in depth order without sorting pairs.
-__global__ void __launch_bounds__(256) depth_key_kernel(int G, const float* __restrict__ depth,
-                                                        std::uint32_t* __restrict__ keys,
-                                                        std::uint32_t* __restrict__ identity) {
-    const int g = blockIdx.x * 256 + threadIdx.x;
-    if (g >= G) return;
-    keys[g] = ordered_bits(depth[g]);
-    identity[g] = static_cast<std::uint32_t>(g);
-}
 
 // Blocks are handed to the eight XCDs round-robin; giving each XCD a contiguous band of tiles keeps the
 // records of a Gaussian that spans neighbouring tiles in one L2.
@@ -752,18 +728,6 @@ int launch_project(hipStream_t s, int G, const float* params, const float* depth
                    TileRect* rects_by_depth, float* record_grads, double* loss, bool first_of_step) {
     hipLaunchKernelGGL(project_kernel, dim3(xad::blocks_for(G, 256)), dim3(256), 0, s, G, params, depth, ordered_depth, rank,
                        status, width, height, records, rects, rects_by_depth, record_grads, loss, first_of_step);
-    XAD_HIP_TRY(hipGetLastError());
-    return XAD_OK;
-}
-
-int launch_depth_rank(hipStream_t s, int G, const std::uint32_t* by_depth, std::uint32_t* rank) {
-    hipLaunchKernelGGL(depth_rank_kernel, dim3(xad::blocks_for(G, 256)), dim3(256), 0, s, G, by_depth, rank);
-    XAD_HIP_TRY(hipGetLastError());
-    return XAD_OK;
-}
-
-int launch_depth_keys(hipStream_t s, int G, const float* depth, std::uint32_t* keys, std::uint32_t* identity) {
-    hipLaunchKernelGGL(depth_key_kernel, dim3(xad::blocks_for(G, 256)), dim3(256), 0, s, G, depth, keys, identity);
     XAD_HIP_TRY(hipGetLastError());
     return XAD_OK;
 }

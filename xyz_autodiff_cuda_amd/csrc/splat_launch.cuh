@@ -27,10 +27,6 @@ enum : int {
 int launch_project(hipStream_t s, int G, const float* params, const float* depth, const float* ordered_depth,
                    const std::uint32_t* rank, std::uint32_t* status, int width, int height, Record* records, TileRect* rects,
                    TileRect* rects_by_depth, float* record_grads, double* loss, bool first_of_step);
-// Depth order: keys[g] = order-preserving bits of depth[g], identity[g] = g; the stable sort of
-// those pairs gives by_depth; rank is its inverse (rank[by_depth[i]] = i).
-int launch_depth_keys(hipStream_t s, int G, const float* depth, std::uint32_t* keys, std::uint32_t* identity);
-int launch_depth_rank(hipStream_t s, int G, const std::uint32_t* by_depth, std::uint32_t* rank);
 
 // Binning (splat_binning.hip): tile lists from tile rectangles, Gaussians taken in the order by_depth.
 constexpr std::uint32_t kBinRangeB = 64;  // list entries a wavefront handles at level B: one per lane
@@ -83,9 +79,13 @@ int render_segments(int width, int height);
 // Also adds the parts of the loss up into loss[0].
 int launch_gaussian_backward(hipStream_t s, int G, const float* params, const float* record_grads, float* grads, double* loss);
 
-// The stable radix sort of (depth bits, index) that yields the depth order (rocPRIM; runs only when a depth changed).
+// The depth order (splat_sort.hip): by_depth = the Gaussians in (depth, index) order, rank its inverse
+// (rank[by_depth[i]] = i), ordered_depth = a copy of depth.  keys_a, keys_b, values_a: G words each of scratch;
+// temp: depth_sort_temp_bytes(G) bytes that are zero before the first sort and are left ready by every sort.
 std::size_t depth_sort_temp_bytes(int G);
-int sort_by_depth(hipStream_t s, void* temp, std::size_t temp_bytes, const std::uint32_t* keys_in,
-                  std::uint32_t* keys_out, const std::uint32_t* values_in, std::uint32_t* values_out, int G);
+std::size_t depth_sort_gave_up_offset();  // byte offset in temp of a word that counts blocks whose bounded wait ran out
+int sort_by_depth(hipStream_t s, void* temp, std::size_t temp_bytes, const float* depth, std::uint32_t* keys_a,
+                  std::uint32_t* keys_b, std::uint32_t* values_a, std::uint32_t* by_depth, std::uint32_t* rank,
+                  float* ordered_depth, int G);
 
 }  // namespace xad_splat

@@ -11,7 +11,7 @@ import warnings
 from . import _lib, rng
 
 PARAM_ROWS = ("cx", "cy", "log_sx", "log_sy", "theta", "r", "g", "b", "opacity")
-STAGES = ("project", "binning", "render_forward", "render_backward", "parameter_backward")
+STAGES = ("sort", "project", "binning", "render_forward", "render_backward", "parameter_backward")
 DEPTH_MODES = {"checked": 0, "static": 1, "every_step": 2}
 
 
@@ -134,6 +134,21 @@ class SplatContext:
         if longest_list:
             out["longest_list"] = longest.value
         return out
+
+
+def depth_order(depth, stream=None):
+    """(order, rank) of a float32 CUDA tensor of depths: order[i] = the i-th element by (depth, index), rank its
+    inverse; int32 tensors holding the unsigned values (xad_depth_order_f32)."""
+    import torch
+
+    _check_tensor(depth, (depth.numel(),), "depth")
+    order = torch.empty(depth.numel(), dtype=torch.int32, device=depth.device)
+    rank = torch.empty_like(order)
+    s = (stream if stream is not None else torch.cuda.current_stream(depth.device)).cuda_stream
+    with torch.cuda.device(depth.device):
+        st = _lib.load().xad_depth_order_f32(depth.numel(), depth.data_ptr(), order.data_ptr(), rank.data_ptr(), s)
+    _lib.check(st, "xad_depth_order_f32")
+    return order, rank
 
 
 def host_step(params, depth, target, width, height, want_grads=True, num_threads=0):
