@@ -61,3 +61,60 @@ def chain_closed_form(inputs):
     ]
     grads = [(-0.5 * w) * d if d is not None else w * (1 - sig) for d in dq]
     return np.stack([w] + grads), q
+
+
+FIELDS = ("cx", "cy", "log_sx", "log_sy", "theta", "r", "g", "b", "opacity")
+
+
+def gradient_distribution(got, fp32_oracle, fp64, mass):
+    """How an implementation's 9 x G gradients sit around the fp64 ones, field by field, beside the same figures
+    for an independent fp32 evaluation (the fp32 oracle).  Errors are in units of `mass` (the sum of the
+    magnitudes of the per-pixel terms behind a gradient: the scale of fp32 rounding in any summation order).
+
+      median, p99      quantiles of |x - fp64| / mass over the Gaussians that reach a pixel, each Gaussian
+                       weighted by its mass: "half (99 %) of the gradient mass sits in entries at least this
+                       accurate".  (Unweighted, the upper quantiles are those of Gaussians hidden behind
+                       others, whose few terms sit next to the 1e-4 stop, where two correct evaluations
+                       differ by the whole term: 1 % of the Gaussians at 200 000, with next to no mass.)
+      bias             sum (x - fp64) / sum mass: an error of one sign (terms left out, a list cut short)
+      along_gradient   sum sign(fp64) (x - fp64) / sum mass: a factor on the gradients (a dropped 1/2, a wrong
+                       constant) has the sign of the gradient even in fields whose gradients sum to nothing
+      flat             fraction of the Gaussians with this gradient within 1e-4 relative
+    """
+    got, fp32_oracle, fp64, mass = (np.asarray(a, np.float64) for a in (got, fp32_oracle, fp64, mass))
+    out = {}
+    for row, field in enumerate(FIELDS):
+        live = mass[row] > 0
+        m, ref = mass[row][live], fp64[row][live]
+        entry = {}
+        for name, x in (("got", got[row][live]), ("fp32_oracle", fp32_oracle[row][live])):
+            e = x - ref
+            relative = np.abs(e) / m
+            order = np.argsort(relative)
+            share = np.cumsum(m[order]) / m.sum()
+            entry[name] = {
+                "median": float(relative[order][np.searchsorted(share, 0.5)]),
+                "p99": float(relative[order][min(np.searchsorted(share, 0.99), relative.size - 1)]),
+                "bias": float(e.sum() / m.sum()), "along_gradient": float((np.sign(ref) * e).sum() / m.sum()),
+                "flat": float((np.abs(e) <= 1e-4 * np.abs(ref)).mean()),
+            }
+        out[field] = entry
+    return out
+
+
+def gradient_distribution_failures(figures, quantile_factor=1.5, bias_limit=2e-6, flat_slack=0.01):
+    """What of gradient_distribution's figures is out of line: quantiles more than quantile_factor times the fp32
+    oracle's own, a bias (plain or along the gradient) beyond bias_limit, or fewer Gaussians within 1e-4
+    relative than the fp32 oracle has (less flat_slack)."""
+    failures = []
+    for field, entry in figures.items():
+        got, ref = entry["got"], entry["fp32_oracle"]
+        for q in ("median", "p99"):
+            if got[q] > quantile_factor * ref[q] + 1e-9:
+                failures.append("%s: %s of |error| / mass %.3g, the fp32 oracle's %.3g" % (field, q, got[q], ref[q]))
+        for b in ("bias", "along_gradient"):
+            if abs(got[b]) > bias_limit:
+                failures.append("%s: %s %.3g (limit %.1g; the fp32 oracle's %.3g)" % (field, b, got[b], bias_limit, ref[b]))
+        if got["flat"] < ref["flat"] - flat_slack:
+            failures.append("%s: %.4f of the Gaussians within 1e-4 relative, the fp32 oracle %.4f" % (field, got["flat"], ref["flat"]))
+    return failures

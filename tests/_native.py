@@ -75,6 +75,21 @@ def eval_logic(name, operands, constants=(), upstream=None, dtype=np.float64, de
     return out[:n_out].copy(), out[n_out:n_out + n_in].copy(), out[n_out + n_in:n].copy()
 
 
+def negligible_in_tile(fields, tiles, device=False):
+    """fields (n, 6) float32: centre x, y, inverse covariance a, b, c, alpha0; tiles (n, 2) float32: the tiles' first
+    pixels.  -> bool array: the entries the compositing kernels would leave out of that tile."""
+    fields = np.ascontiguousarray(fields, np.float32)
+    tiles = np.ascontiguousarray(tiles, np.float32)
+    n = fields.shape[0]
+    assert fields.shape == (n, 6) and tiles.shape == (n, 2)
+    out = np.zeros(n, np.int32)
+    fn = load().xad_test_negligible_in_tile
+    fn.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]
+    rc = fn(1 if device else 0, n, fields.ctypes.data, tiles.ctypes.data, out.ctypes.data)
+    assert rc == 0, rc
+    return out.astype(bool)
+
+
 def parallel_accumulation(threads, block):
     out = np.zeros(3, np.float64)
     rc = load().xad_test_parallel_accumulation(ctypes.c_size_t(threads), ctypes.c_int(block), out.ctypes.data_as(ctypes.c_void_p))

@@ -12,6 +12,7 @@
 #include <xyz_autodiff/util/hip_managed_ptr.cuh>
 #include "tester_suite.cuh"
 #include "concept_checks.cuh"
+#include "../../xyz_autodiff_cuda_amd/csrc/splat_staged.cuh"
 
 using namespace xyz_autodiff;
 
@@ -165,6 +166,26 @@ __global__ void managed_accumulation_kernel(T* values, T* grads, std::size_t thr
 
 bool ok(hipError_t e) { return e == hipSuccess; }
 
+// The test that leaves a list entry out of a tile's compositing (csrc/splat_staged.cuh), on n (record, tile)
+// pairs; fields: n x 6 floats (centre x, y; inverse covariance a, b, c; alpha0), tiles: n x 2 floats (the
+// tile's first pixel).
+XAD_HD int negligible_pair(const float* fields, const float* tiles, int i) {
+    xad_splat::Record record{};
+    record.cx = fields[6 * i];
+    record.cy = fields[6 * i + 1];
+    record.a = fields[6 * i + 2];
+    record.b = fields[6 * i + 3];
+    record.c = fields[6 * i + 4];
+    record.alpha0 = fields[6 * i + 5];
+    const xad_splat::Staged staged = xad_splat::stage_record(&record, 0);
+    return xad_splat::negligible_in_tile(staged, tiles[2 * i], tiles[2 * i + 1]) ? 1 : 0;
+}
+
+__global__ void negligible_kernel(int n, const float* fields, const float* tiles, int* out) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) out[i] = negligible_pair(fields, tiles, i);
+}
+
 template <typename T>
 int managed_accumulation(std::size_t threads, double* out2) {
     auto values = makeHipManagedArray<T>(2);
@@ -194,6 +215,27 @@ extern "C" int xad_test_tester_suite_device(char* text, std::size_t capacity, un
 }
 
 extern "C" int xad_test_case_capacity(void) { return xad_test::kCaseCapacity; }
+
+// side: 0 host, 1 device.  out: n ints, 1 where the entry would be left out.
+extern "C" int xad_test_negligible_in_tile(int side, int n, const float* fields, const float* tiles, int* out) {
+    if (side == 0) {
+        for (int i = 0; i < n; ++i) out[i] = negligible_pair(fields, tiles, i);
+        return 0;
+    }
+    float *d_fields = nullptr, *d_tiles = nullptr;
+    int* d_out = nullptr;
+    if (!ok(hipMalloc(&d_fields, sizeof(float) * 6 * n)) || !ok(hipMalloc(&d_tiles, sizeof(float) * 2 * n)) ||
+        !ok(hipMalloc(&d_out, sizeof(int) * n)))
+        return -2;
+    (void)hipMemcpy(d_fields, fields, sizeof(float) * 6 * n, hipMemcpyHostToDevice);
+    (void)hipMemcpy(d_tiles, tiles, sizeof(float) * 2 * n, hipMemcpyHostToDevice);
+    hipLaunchKernelGGL(negligible_kernel, dim3((n + 255) / 256), dim3(256), 0, 0, n, d_fields, d_tiles, d_out);
+    const int rc = ok(hipDeviceSynchronize()) && ok(hipMemcpy(out, d_out, sizeof(int) * n, hipMemcpyDeviceToHost)) ? 0 : -2;
+    (void)hipFree(d_fields);
+    (void)hipFree(d_tiles);
+    (void)hipFree(d_out);
+    return rc;
+}
 
 extern "C" int xad_test_run_case_host(int id, double* out) { return xad_test::run_case(id, out); }
 

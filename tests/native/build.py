@@ -16,6 +16,8 @@ def source_digest():
     files = [os.path.join(HERE, f) for f in os.listdir(HERE) if f.endswith((".hip", ".cuh", ".inc", ".cpp"))]
     for dirpath, _, names in os.walk(os.path.join(ROOT, "include")):
         files += [os.path.join(dirpath, f) for f in names if f.endswith((".cuh", ".h"))]
+    # the compositing kernels' visibility test, which the tier runs on both sides
+    files += [os.path.join(ROOT, "xyz_autodiff_cuda_amd", "csrc", f) for f in ("splat_staged.cuh", "splat.cuh")]
     for path in sorted(files):
         h.update(os.path.relpath(path, ROOT).encode() + b"\0")
         with open(path, "rb") as f:

@@ -24,7 +24,7 @@ meets the flat figures, 1e-5 relative for forward values and 1e-4 relative for g
 import numpy as np
 import pytest
 
-from tests._metrics import abs_or_rel, covariance_condition
+from tests._metrics import abs_or_rel, covariance_condition, gradient_distribution, gradient_distribution_failures
 
 pytestmark = [pytest.mark.gpu, pytest.mark.timeout(600)]
 
@@ -164,12 +164,26 @@ def _splat_case(gpu, oracle, G, W, H, scale_px, opacity_shift=0.0):
         "pixels_within_1e-5": float((np.abs(got_image - o64["image"]) <= 1e-5).mean()),
     }
     _say("splat %d Gaussians %dx%d" % (G, W, H), **figures)
+    # the same errors in distribution, field by field, beside the fp32 oracle's own
+    distribution = gradient_distribution(got, o32["grads"], o64["grads"], o64["grad_mass"])
+    for field, entry in distribution.items():
+        _say("splat %d Gaussians %dx%d, d/d %s" % (G, W, H, field), **{"%s_%s" % (who, k): v for who in entry for k, v in entry[who].items()})
+    figures["distribution_failures"] = gradient_distribution_failures(distribution)
     assert image_err["over_bound"] <= 1.0, (image_err, figures)
     assert figures["pixels_within_1e-5"] > 0.9999, figures
     assert loss_err["vs_fp32"] <= 1e-6 and loss_err["vs_fp64"] <= 1e-6, (loss_err, figures)
     worst = np.unravel_index(excess.argmax(), excess.shape)
     assert within.all(), ("Gaussians outside |gpu - fp64| <= 1e-4 mass + bound: %d of %d; worst row %d, Gaussian %d" %
                           (int((~within).sum()), G, worst[0], worst[1]), figures)
+    # The allowance above is wide where fp32 itself is poor (it has to hold for every entry), so a small systematic
+    # error would fit under it.  In distribution there is no such room: per field the median and the 99th
+    # percentile of the error (by gradient mass) may be at most 1.5 times the fp32 oracle's own, the errors must
+    # not lean one way (2e-6 of the mass, plain or along the gradient: measured 6e-7 at 200 000 Gaussians, where
+    # the rounding of the one constant -log2(e)/2 in every exponent leans all of them the same way, 8e-8 at
+    # 10 000; a factor of 1.005 on the gradients leans 5e-4), and at least as many Gaussians as in the fp32
+    # oracle must meet the flat 1e-4 relative.
+    assert not figures["distribution_failures"], figures["distribution_failures"]
+    assert figures["gaussians_with_all_gradients_within_1e-4_relative"] >= figures["fp32_oracle_same_figure"] - 0.01, figures
     return figures
 
 
