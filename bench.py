@@ -31,9 +31,10 @@ N_FULL = 64 * 1024 * 1024
 # `bench.py --counter-probe splat` / `--counter-probe splat4` (TCC_ATOMIC_sum per kernel, summed over the
 # iteration's kernels); constants from those profiles, not readings of this run.
 ATOMIC_TRAFFIC = {
-    "config5_200k_2048": {"l2_atomic_requests_measured": 3_665_995, "pairs_in_that_run": 5_484_589,
-                          "values_added": 39_000_000,
-                          "source": "profiles/splat_200k_2048_kernel_counters.md (TCC_ATOMIC_sum: render_backward_kernel 3 665 877, scans 118)"},
+    "config4_10k_512": {"l2_atomic_requests_measured": 132_498, "pairs_in_that_run": 129_843,
+                        "source": "profiles/splat_10k_512_kernel_counters.md (TCC_ATOMIC_sum: render_backward_kernel 132 490, scans 8)"},
+    "config5_200k_2048": {"l2_atomic_requests_measured": 3_666_035, "pairs_in_that_run": 5_500_959,
+                          "source": "profiles/splat_200k_2048_kernel_counters.md (TCC_ATOMIC_sum: render_backward_kernel 3 665 877, scans 158)"},
 }
 
 
@@ -381,10 +382,10 @@ def main():
     ap.add_argument("--n", type=int, default=N_FULL, help="problems per step (default: the full 64 Mi)")
     ap.add_argument("--seed", type=int, default=1234)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs (profiling runs)")
-    ap.add_argument("--counter-probe", choices=("chain", "accumulate", "splat"), default=None,
+    ap.add_argument("--counter-probe", choices=("chain", "accumulate", "splat", "splat4"), default=None,
                     help="launch a few kernels of one leg and exit, for rocprofv3 --pmc runs: chain = a 256 Mi-float "
                          "copy then three chain passes; accumulate = naive and staged accumulation at 64, 4096 and 262144 slots; "
-                         "splat = two iterations of the 200k-Gaussian step")
+                         "splat = two iterations of the 200k-Gaussian step; splat4 = two of the 10k-Gaussian step")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (got --gpus %d)" % args.gpus)
@@ -425,18 +426,18 @@ def main():
         torch.cuda.synchronize()
         print(json.dumps({"counter_probe": "accumulate", "n": m, "order": "per slots in (64, 4096, 262144): global_atomics, auto, wave_lds"}))
         return
-    if args.counter_probe == "splat":
+    if args.counter_probe in ("splat", "splat4"):
         from xyz_autodiff_cuda_amd import splat
 
         del ins, outs
-        G, W, H, scale = 200_000, 2048, 2048, (0.5, 40.0)
+        G, W, H, scale = (200_000, 2048, 2048, (0.5, 40.0)) if args.counter_probe == "splat" else (10_000, 512, 512, (1.0, 20.0))
         target = splat.synthetic_target(G, W, H, seed=77, scale_px=scale, noise=0.02)
         params, depth = splat.synthetic_scene(G, W, H, seed=args.seed, scale_px=scale)
-        ctx = splat.SplatContext(W, H, G, pair_capacity_hint=9_000_000)
+        ctx = splat.SplatContext(W, H, G, pair_capacity_hint=9_000_000 if G > 50_000 else 0)
         for _ in range(2):
             ctx.step(params, depth, target, want_loss=False)
         torch.cuda.synchronize()
-        print(json.dumps({"counter_probe": "splat", "pairs": ctx.stats()["pairs"]}))
+        print(json.dumps({"counter_probe": args.counter_probe, "pairs": ctx.stats()["pairs"]}))
         return
 
     for _ in range(args.warmup):

@@ -97,7 +97,9 @@ int create(const xad_training_config* config, int width, int height, const float
     t->gaussians = config->num_gaussians;
     XAD_HIP_TRY(hipGetDevice(&t->device));
     XAD_HIP_TRY(hipStreamCreate(&t->stream));
-    if (int st = xad_splat_create(width, height, t->gaussians, 0, &t->splat)) return st;
+    // room for Gaussians that grow during training: four times the default (an overflow costs iterations run twice;
+    // the lists take about 16 bytes per pair)
+    if (int st = xad_splat_create(width, height, t->gaussians, static_cast<std::size_t>(t->gaussians) * 32 + 4096, &t->splat)) return st;
     // depth is drawn once and never trained: promise that, so that an iteration never waits for the device
     if (int st = xad_splat_set_depth_mode(t->splat, XAD_SPLAT_DEPTH_STATIC)) return st;
     if (int st = xad_splat_overflow_word(t->splat, &t->overflow_word)) return st;
