@@ -13,6 +13,7 @@ namespace {
 struct HostReport {
     std::uint32_t status[kStatusWords];
     std::uint32_t depth_changed;  // the depth flag as it stood before the binning cleared it
+    std::uint32_t sort_gave_up;   // blocks of the depth sort whose bounded wait ran out (never, on a device of one's own)
     double loss;
 };
 
@@ -173,9 +174,18 @@ int bin_lists(xad_splat_context* c, hipStream_t s, bool clear_depth_flag) {
 int fetch_report(xad_splat_context* c, hipStream_t s) {
     XAD_HIP_TRY(hipMemcpyAsync(c->report->status, c->status, sizeof(std::uint32_t) * kStatusWords, hipMemcpyDeviceToHost, s));
     XAD_HIP_TRY(hipMemcpyAsync(&c->report->loss, c->loss, sizeof(double), hipMemcpyDeviceToHost, s));
+    XAD_HIP_TRY(hipMemcpyAsync(&c->report->sort_gave_up, static_cast<const char*>(c->depth_sort_temp) + depth_sort_gave_up_offset(),
+                               sizeof(std::uint32_t), hipMemcpyDeviceToHost, s));
     XAD_HIP_TRY(hipEventRecord(c->report_ready, s));
     XAD_HIP_TRY(hipEventSynchronize(c->report_ready));
     c->pairs = c->report->status[kStatusPairs];
+    if (c->report->sort_gave_up != 0) {
+        c->order_valid = false;
+        return xad::fail(XAD_ERR_HIP,
+                         "splat: %u blocks of the depth sort gave up waiting for other blocks (is the device shared with work that "
+                         "never ends?); the depth order of the calls since the last report cannot be trusted",
+                         c->report->sort_gave_up);
+    }
     return XAD_OK;
 }
 

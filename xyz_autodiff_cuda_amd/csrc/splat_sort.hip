@@ -36,7 +36,10 @@
 // looks of 8, 16, 24, 32 words 0.071, 0.059-0.064, 0.068, 0.076 ms (more words per look is more code and
 // more registers: with 64 and a wait loop per word a pass spent 20 us fetching instructions); tiles
 // taken by block index instead of by ticket 0.078 (blocks do not start in index order, so more of
-// them wait).  At 10^4 keys (three tiles) 0.05 ms: five launches of about 10 us.
+// them wait).  At 10^4 keys (three tiles) 0.05 ms: five launches of about 10 us.  The five steps in one
+// launch, with a barrier across the (resident) blocks and agent-scope fences between them: 0.23 ms at
+// 2 x 10^5 keys, 0.085 at 10^4 -- the release and acquire of plain data across the XCDs' L2 caches
+// (write back, invalidate) cost far more than the launch boundaries they replace.
 //
 // Equal depths keep index order (every pass is stable and the first one takes the keys in index
 // order).  Order of the keys: the total order of the bit patterns in sign-magnitude reading, with
@@ -170,8 +173,9 @@ __global__ void __launch_bounds__(kSortBlock) sort_pass_kernel(int G, int pass, 
     // the ring: what the pass before this one used is cleared here (by pass 0: what pass 3 of the sort before used)
     if (b == 0 && t < kDigits) {
         const int behind = (pass + kPasses - 1) % kPasses;
-        work[behind * kDigits + t] = 0;
-        if (t == 0) work[kTicketAt + behind] = 0;
+        // (stores that go where the other blocks' atomics go, not through a cached line next to words in use)
+        __hip_atomic_store(work + behind * kDigits + t, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (t == 0) __hip_atomic_store(work + kTicketAt + behind, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
 
     // a wavefront's keys are contiguous; in round i lane l holds key i * 64 + l of them
