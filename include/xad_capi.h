@@ -289,7 +289,7 @@ int xad_adam_step_gated_f32(size_t n, int rows, float* params, const float* grad
  */
 
 /* The fields of TrainingConfig (training_config.h:7-31) with its defaults,
- * followed by the additions of this build (seed, output directory, checkpoints). */
+ * followed by the additions of this build (seed, output directory, checkpoints, image format). */
 typedef struct xad_training_config {
     float lr_center, lr_scale, lr_rotation, lr_color, lr_opacity;
     int max_iterations;   /* 500 */
@@ -304,6 +304,7 @@ typedef struct xad_training_config {
     char output_dir[1024];       /* "output" */
     char checkpoint_path[1024];  /* "" = write none */
     char resume_path[1024];      /* "" = start from random Gaussians */
+    char image_format[8];        /* "jpg" (what the reference writes), "png" or "ppm": the program's snapshots */
 } xad_training_config;
 
 #define XAD_HELP_REQUESTED 4 /* returned by xad_training_config_parse for --help */
@@ -313,8 +314,8 @@ void xad_training_config_defaults(xad_training_config* config);
  * <lr_opacity> then --target PATH, --max-iterations N, --save-interval N,
  * --num-gaussians N, --no-save-images, --beta1 V, --beta2 V, --epsilon V, --help
  * (TrainingConfigParser::parse, training_config.cpp:29-88) and, added here,
- * --seed N, --output-dir DIR, --checkpoint PATH, --checkpoint-interval N,
- * --resume PATH.  Fails like the reference: fewer than five positional
+ * --seed N, --output-dir DIR, --image-format jpg|png|ppm, --checkpoint PATH,
+ * --checkpoint-interval N, --resume PATH.  Fails like the reference: fewer than five positional
  * arguments "Insufficient arguments", an unknown option or an option without
  * its value "Invalid argument", then the checks of validate_config
  * (training_config.cpp:114-146) with its messages. */
@@ -324,13 +325,18 @@ int xad_training_config_validate(const xad_training_config* config);
 const char* xad_training_usage(void);
 
 /* Image files: float RGB in [0, 1], height x width x 3, host memory.
- * xad_image_load reads PNG (not interlaced) or binary PPM/PGM and allocates
- * *rgb (release with xad_image_free); xad_image_save writes 8-bit PNG or PPM by
- * the extension of `path`, quantising like save_image_jpeg (image_utils.cpp:39-56);
+ * xad_image_load (load_image, image_utils.cpp:12-36) reads a PNG, a JPEG
+ * (Huffman-coded, sequential or progressive, grey or colour) or a binary PPM/PGM,
+ * told apart by their first bytes, and allocates *rgb (release with
+ * xad_image_free); xad_image_save writes 8-bit JPEG (quality 90), PNG or PPM by
+ * the extension of `path` (.jpg / .jpeg / .png / .ppm); xad_image_save_jpeg is
+ * save_image_jpeg (image_utils.cpp:38-56; quality 1..100, 90 being its default):
+ * bytes are (unsigned char)(clamped * 255 + 0.5) as there (:42-46);
  * xad_image_test_pattern fills the gradient of create_test_image (:58-77). */
 int xad_image_load(const char* path, int* width, int* height, float** rgb);
 void xad_image_free(float* rgb);
 int xad_image_save(const char* path, int width, int height, const float* rgb);
+int xad_image_save_jpeg(const char* path, int width, int height, const float* rgb, int quality);
 int xad_image_test_pattern(int width, int height, float* rgb);
 
 /* A training run on the current device: parameters, gradients and Adam moments

@@ -167,7 +167,9 @@ int main(int argc, char** argv) {
         std::vector<float> rgb(24 * 10 * 3);
         xad_train::test_pattern(24, 10, rgb.data());
         if (!xad_train::save_image(corpus_dir + "/pattern.png", 24, 10, rgb.data()).empty() ||
-            !xad_train::save_image(corpus_dir + "/pattern.ppm", 24, 10, rgb.data()).empty()) {
+            !xad_train::save_image(corpus_dir + "/pattern.ppm", 24, 10, rgb.data()).empty() ||
+            !xad_train::save_image(corpus_dir + "/pattern.jpg", 24, 10, rgb.data()).empty() ||
+            !xad_train::save_image_jpeg(corpus_dir + "/pattern_q100.jpg", 24, 10, rgb.data(), 100).empty()) {
             std::printf("save_image failed\n");
             return 1;
         }

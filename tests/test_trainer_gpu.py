@@ -313,7 +313,7 @@ def test_command_line_program(gpu, tmp_path):
     target = trainer.test_pattern(96, 64)
     trainer.save_image(tmp_path / "target.png", target)
     args = ["0.2", "0.02", "0.02", "0.02", "0.02", "--target", "target.png", "--num-gaussians", "800", "--max-iterations", "60",
-            "--save-interval", "25", "--output-dir", "out", "--checkpoint", "run.ckpt", "--seed", "3"]
+            "--save-interval", "25", "--output-dir", "out", "--checkpoint", "run.ckpt", "--seed", "3", "--image-format", "png"]
     code, out, err = _run_program(args, tmp_path)
     assert code == 0, err
     losses = [float(x) for x in re.findall(r"average Loss: ([0-9.e+-]+)", out)]
@@ -326,6 +326,22 @@ def test_command_line_program(gpu, tmp_path):
     first = trainer.load_image(tmp_path / "out" / "iteration_000000.png")
     assert np.mean((final - target) ** 2) < 0.5 * np.mean((first - target) ** 2)
     assert "Program completed successfully!" in out and "Checkpoint: run.ckpt (iteration 60)" in out
+
+    # without --image-format: the names and the format of the reference (gaussian_splatting_training.cu:106, :124),
+    # from a JPEG target; another JPEG decoder reads the snapshots and agrees with the trainer's reader
+    from PIL import Image
+
+    trainer.save_image(tmp_path / "target.jpg", target)
+    code, out, err = _run_program(args[:5] + ["--target", "target.jpg", "--num-gaussians", "300", "--max-iterations", "10",
+                                              "--save-interval", "5", "--output-dir", "jpg_out"], tmp_path)
+    assert code == 0, err
+    assert "Target image: 96x64" in out
+    assert sorted(os.listdir(tmp_path / "jpg_out")) == ["iteration_000000.jpg", "iteration_000005.jpg", "iteration_000010.jpg", "target.jpg"]
+    for name in ("iteration_000010.jpg", "target.jpg"):
+        theirs = np.asarray(Image.open(tmp_path / "jpg_out" / name).convert("RGB")).astype(np.int32)
+        ours = np.rint(trainer.load_image(tmp_path / "jpg_out" / name) * 255).astype(np.int32)
+        assert theirs.shape == (64, 96, 3) and np.abs(theirs - ours).max() <= 4
+    assert np.abs(np.asarray(Image.open(tmp_path / "jpg_out" / "target.jpg").convert("RGB")) / 255.0 - target).mean() < 0.02
 
     # resume: continues at iteration 60 and stops at 80
     code, out, err = _run_program(args[:5] + ["--target", "target.png", "--num-gaussians", "800", "--max-iterations", "80", "--no-save-images",

@@ -58,6 +58,7 @@ SIGNATURES = {
     "xad_image_load": [ctypes.c_char_p, ctypes.POINTER(_int), ctypes.POINTER(_int), ctypes.POINTER(_f32p)],
     "xad_image_free": [_f32p],
     "xad_image_save": [ctypes.c_char_p, _int, _int, _vp],
+    "xad_image_save_jpeg": [ctypes.c_char_p, _int, _int, _vp, _int],
     "xad_image_test_pattern": [_int, _int, _vp],
     "xad_trainer_create": [_vp, _int, _int, _vp, ctypes.POINTER(_vp)],
     "xad_trainer_destroy": [_vp],

@@ -2,6 +2,8 @@
 
 #include <zlib.h>
 
+#include "jpeg_codec.h"
+
 #include <algorithm>
 #include <cctype>
 #include <cstdint>
@@ -53,12 +55,12 @@ int paeth(int a, int b, int c) {
     return pb <= pc ? b : c;
 }
 
-// Undoes the per-row prediction filters in place; `raw` holds height rows of
+// Undoes the per-row prediction filters in place; `raw` points at height rows of
 // 1 + row_bytes bytes.  Returns false on an unknown filter type.
-bool unfilter(Bytes& raw, std::size_t height, std::size_t row_bytes, std::size_t bpp) {
+bool unfilter(unsigned char* raw, std::size_t height, std::size_t row_bytes, std::size_t bpp) {
     const Bytes zero_row(row_bytes, 0);
     for (std::size_t y = 0; y < height; ++y) {
-        unsigned char* row = raw.data() + y * (row_bytes + 1) + 1;
+        unsigned char* row = raw + y * (row_bytes + 1) + 1;
         const unsigned char* up = y ? row - (row_bytes + 1) : zero_row.data();
         const int type = row[-1];
         for (std::size_t i = 0; i < row_bytes; ++i) {
@@ -83,7 +85,7 @@ bool unfilter(Bytes& raw, std::size_t height, std::size_t row_bytes, std::size_t
 std::string decode_png(const Bytes& file, Image& out) {
     std::size_t pos = 8;
     std::uint32_t width = 0, height = 0;
-    int depth = 0, colour = -1;
+    int depth = 0, colour = -1, interlaced = 0;
     Bytes palette, compressed;
     bool seen_end = false;
     while (!seen_end) {
@@ -100,7 +102,8 @@ std::string decode_png(const Bytes& file, Image& out) {
             depth = data[8];
             colour = data[9];
             if (data[10] != 0 || data[11] != 0) return "PNG: unknown compression or filter method";
-            if (data[12] != 0) return "PNG: interlaced files are not supported";
+            interlaced = data[12];
+            if (interlaced > 1) return "PNG: unknown interlace method";
         } else if (colour < 0) {
             return "PNG: first chunk is not the header";
         } else if (!std::memcmp(type, "PLTE", 4)) {
@@ -130,38 +133,61 @@ std::string decode_png(const Bytes& file, Image& out) {
     if (width == 0 || height == 0 || std::size_t(width) * height > kMaxPixels) return "PNG: unreasonable image size";
     if (colour == 3 && (palette.empty() || palette.size() % 3)) return "PNG: palette missing or malformed";
 
-    const std::size_t row_bytes = (std::size_t(width) * channels * depth + 7) / 8;
-    Bytes raw(std::size_t(height) * (row_bytes + 1));
+    // The image as one pass, or as the seven passes of Adam7: each pass is a smaller image of the pixels
+    // (x0 + i dx, y0 + j dy), filtered row by row on its own.
+    struct Pass { std::size_t x0, y0, dx, dy; };
+    static const Pass kWhole[1] = {{0, 0, 1, 1}};
+    static const Pass kAdam7[7] = {{0, 0, 8, 8}, {4, 0, 8, 8}, {0, 4, 4, 8}, {2, 0, 4, 4}, {0, 2, 2, 4}, {1, 0, 2, 2}, {0, 1, 1, 2}};
+    const Pass* passes = interlaced ? kAdam7 : kWhole;
+    const int pass_count = interlaced ? 7 : 1;
+    const std::size_t bits_per_pixel = std::size_t(channels) * depth;
+    std::size_t total = 0;
+    for (int p = 0; p < pass_count; ++p) {
+        const std::size_t pw = (width + passes[p].dx - 1 - passes[p].x0) / passes[p].dx;
+        const std::size_t ph = (height + passes[p].dy - 1 - passes[p].y0) / passes[p].dy;
+        if (pw && ph) total += ph * (1 + (pw * bits_per_pixel + 7) / 8);
+    }
+    Bytes raw(total);
     uLongf raw_size = raw.size();
     const int z = uncompress(raw.data(), &raw_size, compressed.data(), compressed.size());
     if (z != Z_OK || raw_size != raw.size()) return "PNG: image data does not inflate to the declared size";
-    if (!unfilter(raw, height, row_bytes, std::max<std::size_t>(1, std::size_t(channels) * depth / 8)))
-        return "PNG: unknown row filter";
 
     out.width = static_cast<int>(width);
     out.height = static_cast<int>(height);
     out.rgb.assign(std::size_t(width) * height * 3, 0.0f);
     const float max_sample = static_cast<float>((1u << depth) - 1);
-    for (std::size_t y = 0; y < height; ++y) {
-        const unsigned char* row = raw.data() + y * (row_bytes + 1) + 1;
-        auto sample = [&](std::size_t index) -> unsigned {
-            if (depth == 8) return row[index];
-            if (depth == 16) return (unsigned(row[2 * index]) << 8) | row[2 * index + 1];
-            const std::size_t bit = index * depth;
-            return (row[bit >> 3] >> (8 - depth - (bit & 7))) & ((1u << depth) - 1);
-        };
-        for (std::size_t x = 0; x < width; ++x) {
-            float* px = &out.rgb[(y * width + x) * 3];
-            if (colour == 3) {
-                const unsigned entry = sample(x);
-                if (3 * entry + 2 >= palette.size()) return "PNG: palette index out of range";
-                for (int c = 0; c < 3; ++c) px[c] = palette[3 * entry + c] / 255.0f;
-            } else if (channels <= 2) {
-                px[0] = px[1] = px[2] = sample(x * channels) / max_sample;
-            } else {
-                for (int c = 0; c < 3; ++c) px[c] = sample(x * channels + c) / max_sample;
+    std::size_t offset = 0;
+    for (int p = 0; p < pass_count; ++p) {
+        const Pass& pass = passes[p];
+        const std::size_t pw = (width + pass.dx - 1 - pass.x0) / pass.dx;
+        const std::size_t ph = (height + pass.dy - 1 - pass.y0) / pass.dy;
+        if (pw == 0 || ph == 0) continue;
+        const std::size_t row_bytes = (pw * bits_per_pixel + 7) / 8;
+        if (!unfilter(raw.data() + offset, ph, row_bytes, std::max<std::size_t>(1, bits_per_pixel / 8)))
+            return "PNG: unknown row filter";
+        for (std::size_t j = 0; j < ph; ++j) {
+            const unsigned char* row = raw.data() + offset + j * (row_bytes + 1) + 1;
+            auto sample = [&](std::size_t index) -> unsigned {
+                if (depth == 8) return row[index];
+                if (depth == 16) return (unsigned(row[2 * index]) << 8) | row[2 * index + 1];
+                const std::size_t bit = index * depth;
+                return (row[bit >> 3] >> (8 - depth - (bit & 7))) & ((1u << depth) - 1);
+            };
+            const std::size_t y = pass.y0 + j * pass.dy;
+            for (std::size_t i = 0; i < pw; ++i) {
+                float* px = &out.rgb[(y * width + pass.x0 + i * pass.dx) * 3];
+                if (colour == 3) {
+                    const unsigned entry = sample(i);
+                    if (3 * entry + 2 >= palette.size()) return "PNG: palette index out of range";
+                    for (int c = 0; c < 3; ++c) px[c] = palette[3 * entry + c] / 255.0f;
+                } else if (channels <= 2) {
+                    px[0] = px[1] = px[2] = sample(i * channels) / max_sample;
+                } else {
+                    for (int c = 0; c < 3; ++c) px[c] = sample(i * channels + c) / max_sample;
+                }
             }
         }
+        offset += ph * (row_bytes + 1);
     }
     return "";
 }
@@ -264,19 +290,37 @@ std::string load_image(const std::string& path, Image& out) {
     if (std::string err = read_file(path, file); !err.empty()) return err;
     if (file.size() >= 8 && !std::memcmp(file.data(), kPngSignature, 8)) return decode_png(file, out);
     if (file.size() >= 3 && file[0] == 'P' && (file[1] == '6' || file[1] == '5')) return decode_netpbm(file, out);
-    if (file.size() >= 2 && file[0] == 0xFF && file[1] == 0xD8) return "JPEG files are not supported; convert " + path + " to PNG or PPM";
-    return path + " is neither a PNG nor a binary PPM/PGM file";
+    if (file.size() >= 2 && file[0] == 0xFF && file[1] == 0xD8) return decode_jpeg(file, out);
+    return path + " is neither a PNG, a JPEG nor a binary PPM/PGM file";
 }
 
-std::string save_image(const std::string& path, int width, int height, const float* rgb) {
+namespace {
+
+// byte = (unsigned char)(clamped * 255 + 0.5), as image_utils.cpp:42-46 quantises before its encoder
+std::string to_bytes(int width, int height, const float* rgb, Bytes& pixels) {
     if (width <= 0 || height <= 0 || !rgb) return "save_image: empty image";
-    Bytes pixels(std::size_t(width) * height * 3);
+    pixels.resize(std::size_t(width) * height * 3);
     for (std::size_t i = 0; i < pixels.size(); ++i) {
         const float v = rgb[i];
         const float clamped = v > 0.0f ? (v < 1.0f ? v : 1.0f) : 0.0f;  // NaN becomes 0
         pixels[i] = static_cast<unsigned char>(clamped * 255.0f + 0.5f);
     }
-    Bytes file;
+    return "";
+}
+
+}  // namespace
+
+std::string save_image_jpeg(const std::string& path, int width, int height, const float* rgb, int quality) {
+    Bytes pixels, file;
+    if (std::string err = to_bytes(width, height, rgb, pixels); !err.empty()) return err;
+    if (std::string err = encode_jpeg(width, height, pixels, quality, file); !err.empty()) return err;
+    return write_file(path, file);
+}
+
+std::string save_image(const std::string& path, int width, int height, const float* rgb) {
+    if (ends_with(path, ".jpg") || ends_with(path, ".jpeg")) return save_image_jpeg(path, width, height, rgb, kDefaultJpegQuality);
+    Bytes pixels, file;
+    if (std::string err = to_bytes(width, height, rgb, pixels); !err.empty()) return err;
     if (ends_with(path, ".png")) {
         if (std::string err = encode_png(width, height, pixels, file); !err.empty()) return err;
     } else if (ends_with(path, ".ppm")) {
@@ -285,7 +329,7 @@ std::string save_image(const std::string& path, int width, int height, const flo
         file.assign(header, header + n);
         file.insert(file.end(), pixels.begin(), pixels.end());
     } else {
-        return "save_image: " + path + " must end in .png or .ppm";
+        return "save_image: " + path + " must end in .jpg, .jpeg, .png or .ppm";
     }
     return write_file(path, file);
 }

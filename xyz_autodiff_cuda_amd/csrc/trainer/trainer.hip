@@ -364,6 +364,15 @@ extern "C" int xad_image_save(const char* path, int width, int height, const flo
     return XAD_OK;
 }
 
+extern "C" int xad_image_save_jpeg(const char* path, int width, int height, const float* rgb, int quality) {
+    XAD_REQUIRE(path && rgb, "path and rgb must not be null");
+    XAD_REQUIRE(width > 0 && height > 0, "image size must be positive, got %d x %d", width, height);
+    XAD_REQUIRE(quality >= 1 && quality <= 100, "JPEG quality must be within 1..100, got %d", quality);
+    const std::string err = xad_train::save_image_jpeg(path, width, height, rgb, quality);
+    XAD_REQUIRE(err.empty(), "%s", err.c_str());
+    return XAD_OK;
+}
+
 extern "C" int xad_image_test_pattern(int width, int height, float* rgb) {
     XAD_REQUIRE(rgb, "rgb must not be null");
     XAD_REQUIRE(width > 0 && height > 0, "image size must be positive, got %d x %d", width, height);

@@ -2,7 +2,7 @@
 // messages of TrainingConfigParser in xyz-autodiff-cuda
 // (examples/mini-gaussian-splatting/training_config.cpp:29-146), returned as
 // status codes and error text instead of exceptions, plus the options this
-// build adds (seed, output directory, checkpoints).
+// build adds (seed, output directory, image format, checkpoints).
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -23,7 +23,7 @@ const char kUsage[] =
     "  lr_opacity     Learning rate for Gaussian opacity parameters\n"
     "\n"
     "Options:\n"
-    "  --target PATH              Target image file path, PNG or PPM (required)\n"
+    "  --target PATH              Target image file path, JPEG, PNG or PPM (required)\n"
     "  --max-iterations N         Maximum training iterations (default: 500)\n"
     "  --save-interval N          Save image every N iterations (default: 25)\n"
     "  --num-gaussians N          Number of Gaussians to use (default: 1000)\n"
@@ -33,6 +33,7 @@ const char kUsage[] =
     "  --epsilon VALUE            Adam optimizer epsilon parameter (default: 1e-8)\n"
     "  --seed N                   Seed of the initial Gaussians (default: 0)\n"
     "  --output-dir DIR           Where images are written (default: output)\n"
+    "  --image-format FORMAT      jpg, png or ppm: the format of those images (default: jpg)\n"
     "  --checkpoint PATH          Write the training state to PATH at the end\n"
     "  --checkpoint-interval N    ... and every N iterations\n"
     "  --resume PATH              Continue from the checkpoint at PATH\n"
@@ -65,6 +66,7 @@ extern "C" void xad_training_config_defaults(xad_training_config* c) {
     c->seed = 0;
     c->checkpoint_interval = 0;
     std::strcpy(c->output_dir, "output");
+    std::strcpy(c->image_format, "jpg");
 }
 
 extern "C" int xad_training_config_validate(const xad_training_config* c) {
@@ -82,6 +84,8 @@ extern "C" int xad_training_config_validate(const xad_training_config* c) {
     XAD_REQUIRE(c->checkpoint_interval == 0 || c->checkpoint_path[0] != '\0',
                 "A checkpoint interval needs a checkpoint path (--checkpoint)");
     XAD_REQUIRE(c->output_dir[0] != '\0', "Output directory must not be empty");
+    XAD_REQUIRE(!std::strcmp(c->image_format, "jpg") || !std::strcmp(c->image_format, "png") || !std::strcmp(c->image_format, "ppm"),
+                "Image format must be jpg, png or ppm");
     return XAD_OK;
 }
 
@@ -121,6 +125,10 @@ extern "C" int xad_training_config_parse(int argc, const char* const* argv, xad_
             c->seed = std::strtoull(argv[++at], nullptr, 10);
         } else if (arg == "--output-dir" && has_value) {
             path_ok = copy_path(c->output_dir, argv[++at]);
+        } else if (arg == "--image-format" && has_value) {
+            const char* format = argv[++at];
+            XAD_REQUIRE(std::strlen(format) < sizeof c->image_format, "Image format must be jpg, png or ppm");
+            std::strcpy(c->image_format, format);
         } else if (arg == "--checkpoint" && has_value) {
             path_ok = copy_path(c->checkpoint_path, argv[++at]);
         } else if (arg == "--checkpoint-interval" && has_value) {

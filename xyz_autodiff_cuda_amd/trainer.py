@@ -31,6 +31,7 @@ class TrainingConfig(ctypes.Structure):
         ("output_dir", ctypes.c_char * 1024),
         ("checkpoint_path", ctypes.c_char * 1024),
         ("resume_path", ctypes.c_char * 1024),
+        ("image_format", ctypes.c_char * 8),
     ]
 
     @classmethod
@@ -76,11 +77,16 @@ def load_image(path):
         lib.xad_image_free(data)
 
 
-def save_image(path, rgb):
+def save_image(path, rgb, quality=None):
+    """By the extension of `path` (.jpg / .jpeg / .png / .ppm); with a quality (1..100), a JPEG whatever the extension."""
     rgb = np.ascontiguousarray(rgb, dtype=np.float32)
     if rgb.ndim != 3 or rgb.shape[2] != 3:
         raise ValueError("expected an array of shape (height, width, 3)")
-    _lib.check(_lib.load().xad_image_save(os.fsencode(path), rgb.shape[1], rgb.shape[0], rgb.ctypes.data_as(ctypes.c_void_p)), "xad_image_save")
+    lib, data = _lib.load(), rgb.ctypes.data_as(ctypes.c_void_p)
+    if quality is None:
+        _lib.check(lib.xad_image_save(os.fsencode(path), rgb.shape[1], rgb.shape[0], data), "xad_image_save")
+    else:
+        _lib.check(lib.xad_image_save_jpeg(os.fsencode(path), rgb.shape[1], rgb.shape[0], data, int(quality)), "xad_image_save_jpeg")
 
 
 def test_pattern(width, height):
