@@ -326,8 +326,8 @@ const char* xad_training_usage(void);
 
 /* Image files: float RGB in [0, 1], height x width x 3, host memory.
  * xad_image_load (load_image, image_utils.cpp:12-36) reads a PNG, a JPEG
- * (Huffman-coded, sequential or progressive, grey or colour) or a binary PPM/PGM,
- * told apart by their first bytes, and allocates *rgb (release with
+ * (Huffman-coded, sequential or progressive, grey or colour), an uncompressed
+ * BMP or a binary PPM/PGM, told apart by their first bytes, and allocates *rgb (release with
  * xad_image_free); xad_image_save writes 8-bit JPEG (quality 90), PNG or PPM by
  * the extension of `path` (.jpg / .jpeg / .png / .ppm); xad_image_save_jpeg is
  * save_image_jpeg (image_utils.cpp:38-56; quality 1..100, 90 being its default):

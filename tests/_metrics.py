@@ -102,15 +102,17 @@ def gradient_distribution(got, fp32_oracle, fp64, mass):
     return out
 
 
-def gradient_distribution_failures(figures, quantile_factor=1.5, bias_limit=2e-6, flat_slack=0.01):
+def gradient_distribution_failures(figures, quantile_factor=1.5, bias_limit=2e-6, flat_slack=0.01, quantile_floor=1e-9):
     """What of gradient_distribution's figures is out of line: quantiles more than quantile_factor times the fp32
-    oracle's own, a bias (plain or along the gradient) beyond bias_limit, or fewer Gaussians within 1e-4
-    relative than the fp32 oracle has (less flat_slack)."""
+    oracle's own (plus quantile_floor: two fp32 evaluations of a few thousand Gaussians have medians of 1e-8 to 1e-7
+    of the mass, below the 6e-8 an fp32 value resolves, and these vary by a factor of two from run to run with the
+    order of the threads' sums), a bias (plain or along the gradient) beyond bias_limit, or fewer Gaussians within
+    1e-4 relative than the fp32 oracle has (less flat_slack)."""
     failures = []
     for field, entry in figures.items():
         got, ref = entry["got"], entry["fp32_oracle"]
         for q in ("median", "p99"):
-            if got[q] > quantile_factor * ref[q] + 1e-9:
+            if got[q] > quantile_factor * ref[q] + quantile_floor:
                 failures.append("%s: %s of |error| / mass %.3g, the fp32 oracle's %.3g" % (field, q, got[q], ref[q]))
         for b in ("bias", "along_gradient"):
             if abs(got[b]) > bias_limit:

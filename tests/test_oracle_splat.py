@@ -301,7 +301,9 @@ def test_the_distribution_checks_pass_an_honest_evaluation_and_catch_a_small_sys
     order, own exp and sincos) passes; gradients that are 0.5 % too large, or that lean one way by 5e-6 of
     their mass, or in which one Gaussian in fifty lost its contributions, do not.  (The factor on the quantiles is
     the full-size tests' 1.5 on the well-conditioned recipe; on these few thousand anisotropic Gaussians the 99th
-    percentile hangs on a handful of heavy ones and two honest evaluations differ by up to 2 in it.)"""
+    percentile hangs on a handful of heavy ones and two honest evaluations differ by up to 2 in it, and the medians
+    lie below what fp32 resolves, so they get a floor of 1e-7 of the mass: both evaluations sum in the order their
+    threads happen to take, and without the floor one run in thirty or so fell outside.)"""
     from tests._metrics import gradient_distribution, gradient_distribution_failures
     from xyz_autodiff_cuda_amd import splat
 
@@ -311,7 +313,7 @@ def test_the_distribution_checks_pass_an_honest_evaluation_and_catch_a_small_sys
 
     def failures(got):
         return gradient_distribution_failures(gradient_distribution(got, o32["grads"], o64["grads"], o64["grad_mass"]),
-                                              quantile_factor=quantile_factor)
+                                              quantile_factor=quantile_factor, quantile_floor=1e-7)
 
     assert failures(honest) == []
     g32 = o32["grads"].astype(np.float64)

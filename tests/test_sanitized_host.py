@@ -62,6 +62,11 @@ def _corpus(directory):
     buffer = io.BytesIO()
     Image.fromarray(smooth[:, :, 0]).save(buffer, "JPEG", quality=60, progressive=True)
     files["grey_progressive.jpg"] = buffer.getvalue()
+    for name, image in {"rgb.bmp": Image.fromarray(rgb), "palette.bmp": Image.fromarray(rgb).quantize(colors=16),
+                        "bilevel.bmp": Image.fromarray(rgb[:, :, 0]).convert("1"), "rgba.bmp": Image.fromarray(np.dstack([rgb, rgb[:, :, :1]]))}.items():
+        buffer = io.BytesIO()
+        image.save(buffer, "BMP")
+        files[name] = buffer.getvalue()
     for name, data in files.items():
         with open(os.path.join(directory, name), "wb") as f:
             f.write(data)

@@ -297,6 +297,89 @@ def test_test_pattern(xad):
     np.testing.assert_array_equal(got[:, :, 2], np.float32(0.5) * (x + y))
 
 
+# ---- BMP ------------------------------------------------------------------------------
+
+def _bmp(width, height, bits, rows, palette=b"", compression=0, masks=b"", top_down=False, core=False):
+    """rows: top-to-bottom list of unpadded row bytes."""
+    padded = [r + bytes(-len(r) % 4) for r in (rows if top_down else rows[::-1])]
+    if core:
+        info = struct.pack("<IHHHH", 12, width, height, 1, bits)
+    else:
+        info = struct.pack("<IiiHHIIiiII", 40, width, -height if top_down else height, 1, bits, compression, 0, 2835, 2835,
+                           len(palette) // 4, 0)
+    offset = 14 + len(info) + len(masks) + len(palette)
+    body = b"".join(padded)
+    return b"BM" + struct.pack("<IHHI", offset + len(body), 0, 0, offset) + info + masks + palette + body
+
+
+def test_bmp_reader_against_pillow(xad, tmp_path):
+    from PIL import Image
+
+    rng = np.random.default_rng(11)
+    rgb = rng.integers(0, 256, (9, 13, 3), dtype=np.uint8)  # 13 x 3 bytes per row: padding is exercised
+    images = {"rgb": Image.fromarray(rgb), "grey": Image.fromarray(rgb[:, :, 0]),
+              "palette": Image.fromarray(rgb).quantize(colors=37), "bilevel": Image.fromarray(rgb[:, :, 1]).convert("1"),
+              "rgba": Image.fromarray(np.dstack([rgb, rgb[:, :, :1]]))}
+    for name, image in images.items():
+        path = tmp_path / (name + ".bmp")
+        image.save(path, "BMP")
+        want = np.asarray(Image.open(path).convert("RGB")).astype(np.float32) / np.float32(255)
+        np.testing.assert_array_equal(trainer.load_image(path), want, err_msg=name)
+
+
+def test_bmp_reader_layouts(xad, tmp_path):
+    rng = np.random.default_rng(12)
+    h, w = 5, 7
+    rgb = rng.integers(0, 256, (h, w, 3), dtype=np.uint8)
+    want = rgb.astype(np.float32) / np.float32(255)
+    bgr_rows = [rgb[y, :, ::-1].tobytes() for y in range(h)]
+    for name, data in {"bottom_up": _bmp(w, h, 24, bgr_rows), "top_down": _bmp(w, h, 24, bgr_rows, top_down=True),
+                       "core": _bmp(w, h, 24, bgr_rows, core=True)}.items():
+        (tmp_path / (name + ".bmp")).write_bytes(data)
+        np.testing.assert_array_equal(trainer.load_image(tmp_path / (name + ".bmp")), want, err_msg=name)
+    # 4 bits per pixel with a colour table of 11 entries (blue, green, red, unused)
+    table = rng.integers(0, 256, (11, 4), dtype=np.uint8)
+    index = rng.integers(0, 11, (h, w))
+    rows = [bytes((int(a) << 4) | int(b) for a, b in zip(list(r[0::2]), list(r[1::2]) + [0])) for r in index]
+    (tmp_path / "p4.bmp").write_bytes(_bmp(w, h, 4, rows, palette=table.tobytes()))
+    np.testing.assert_array_equal(trainer.load_image(tmp_path / "p4.bmp"), table[index][:, :, 2::-1].astype(np.float32) / np.float32(255))
+    # 16 bits: five bits a channel by default, 5-6-5 by masks; 32 bits with masks in another order
+    r5, g6, b5 = rng.integers(0, 32, (h, w)), rng.integers(0, 64, (h, w)), rng.integers(0, 32, (h, w))
+    rows = [((r5[y] << 10) | ((g6[y] >> 1) << 5) | b5[y]).astype("<u2").tobytes() for y in range(h)]
+    (tmp_path / "x555.bmp").write_bytes(_bmp(w, h, 16, rows))
+    want555 = np.stack([r5 / 31, (g6 >> 1) / 31, b5 / 31], axis=2).astype(np.float32)
+    np.testing.assert_allclose(trainer.load_image(tmp_path / "x555.bmp"), want555, rtol=0, atol=1e-7)
+    rows = [((r5[y] << 11) | (g6[y] << 5) | b5[y]).astype("<u2").tobytes() for y in range(h)]
+    (tmp_path / "r565.bmp").write_bytes(_bmp(w, h, 16, rows, compression=3, masks=struct.pack("<III", 0xF800, 0x07E0, 0x001F)))
+    want565 = np.stack([r5 / 31, g6 / 63, b5 / 31], axis=2).astype(np.float32)
+    np.testing.assert_allclose(trainer.load_image(tmp_path / "r565.bmp"), want565, rtol=0, atol=1e-7)
+    packed = (rgb[:, :, 0].astype(np.uint32) << 8) | (rgb[:, :, 1].astype(np.uint32) << 24) | (rgb[:, :, 2].astype(np.uint32) << 16)
+    (tmp_path / "masks32.bmp").write_bytes(_bmp(w, h, 32, [packed[y].astype("<u4").tobytes() for y in range(h)], compression=3,
+                                                masks=struct.pack("<III", 0x0000FF00, 0xFF000000, 0x00FF0000)))
+    np.testing.assert_array_equal(trainer.load_image(tmp_path / "masks32.bmp"), want)
+
+
+def test_bmp_reader_rejects_damage(xad, tmp_path):
+    rgb = np.random.default_rng(13).integers(0, 256, (4, 4, 3), dtype=np.uint8)
+    rows = [rgb[y].tobytes() for y in range(4)]
+    good = _bmp(4, 4, 24, rows)
+    table = bytes(range(16))  # four entries
+    cases = {
+        "run_length": (_bmp(4, 4, 8, [bytes(4)] * 4, palette=table, compression=1), "compressed"),
+        "short": (good[:-5], "shorter"),
+        "depth": (_bmp(4, 4, 7, rows), "bit depth"),
+        "empty": (_bmp(0, 4, 24, rows), "size"),
+        "huge": (_bmp(70000, 70000, 24, rows), "size"),
+        "index": (_bmp(4, 4, 8, [bytes([0, 1, 2, 9])] * 4, palette=table), "colour index"),
+        "table": (_bmp(4, 4, 8, [bytes(4)] * 4, palette=table)[:60], "colour table"),
+        "header": (b"BM" + bytes(12) + struct.pack("<I", 13) + bytes(40), "header"),
+    }
+    for name, (data, message) in cases.items():
+        (tmp_path / (name + ".bmp")).write_bytes(data)
+        with pytest.raises(xad.XadError, match=message):
+            trainer.load_image(tmp_path / (name + ".bmp"))
+
+
 # ---- JPEG -----------------------------------------------------------------------------
 
 def _scene(width, height, seed):

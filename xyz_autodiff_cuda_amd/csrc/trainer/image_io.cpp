@@ -275,6 +275,95 @@ std::string decode_netpbm(const Bytes& file, Image& out) {
     return "";
 }
 
+// ---- BMP -----------------------------------------------------------------------
+
+std::uint32_t le32(const unsigned char* p) {
+    return std::uint32_t(p[0]) | (std::uint32_t(p[1]) << 8) | (std::uint32_t(p[2]) << 16) | (std::uint32_t(p[3]) << 24);
+}
+
+std::uint32_t le16(const unsigned char* p) { return std::uint32_t(p[0]) | (std::uint32_t(p[1]) << 8); }
+
+// The field of a packed pixel that a mask selects, as a fraction of the field's largest value.
+float masked_field(std::uint32_t value, std::uint32_t mask) {
+    if (mask == 0) return 0.0f;
+    int shift = 0;
+    while (!((mask >> shift) & 1u)) ++shift;
+    return static_cast<float>((value & mask) >> shift) / static_cast<float>(mask >> shift);
+}
+
+// Windows bitmaps without compression: 1, 4 or 8 bits with a colour table, 16 or 32 bits with the default or
+// given channel masks, 24 bits; rows bottom-up or (negative height) top-down, padded to four bytes.
+std::string decode_bmp(const Bytes& file, Image& out) {
+    if (file.size() < 26) return "BMP: truncated file";
+    const std::size_t data_offset = le32(&file[10]);
+    const std::size_t header = le32(&file[14]);
+    long long width, height;
+    unsigned bits, compression = 0, colours = 0;
+    std::size_t entry_bytes = 4;
+    if (header == 12) {
+        width = le16(&file[18]);
+        height = le16(&file[20]);
+        bits = le16(&file[24]);
+        entry_bytes = 3;
+    } else if (header >= 40 && header <= 256 && file.size() >= 14 + header) {
+        width = static_cast<std::int32_t>(le32(&file[18]));
+        height = static_cast<std::int32_t>(le32(&file[22]));
+        bits = le16(&file[28]);
+        compression = le32(&file[30]);
+        colours = le32(&file[46]);
+    } else {
+        return "BMP: unknown header";
+    }
+    const bool top_down = height < 0;
+    if (top_down) height = -height;
+    if (width <= 0 || height <= 0 || static_cast<unsigned long long>(width) * static_cast<unsigned long long>(height) > kMaxPixels)
+        return "BMP: unreasonable image size";
+    if (bits != 1 && bits != 4 && bits != 8 && bits != 16 && bits != 24 && bits != 32) return "BMP: unknown bit depth";
+    const bool given_masks = compression == 3 || compression == 6;
+    if (compression != 0 && !(given_masks && (bits == 16 || bits == 32))) return "BMP: compressed files are not supported";
+    std::uint32_t mask[3] = {0x00FF0000u, 0x0000FF00u, 0x000000FFu};
+    if (bits == 16) mask[0] = 0x7C00u, mask[1] = 0x03E0u, mask[2] = 0x001Fu;
+    if (given_masks) {
+        if (file.size() < 66) return "BMP: truncated file";
+        for (int c = 0; c < 3; ++c) mask[c] = le32(&file[54 + 4 * c]);
+        if (bits == 16)
+            for (std::uint32_t& m : mask) m &= 0xFFFFu;
+    }
+    std::size_t entries = 0;
+    const unsigned char* table = nullptr;
+    if (bits <= 8) {
+        entries = colours ? colours : (std::size_t(1) << bits);
+        if (entries > 256) return "BMP: colour table too large";
+        const std::size_t table_offset = 14 + header;
+        if (table_offset > file.size() || entries * entry_bytes > file.size() - table_offset) return "BMP: truncated colour table";
+        table = &file[table_offset];
+    }
+    const std::size_t row_bytes = (static_cast<std::size_t>(width) * bits + 31) / 32 * 4;
+    if (data_offset > file.size() || row_bytes * static_cast<std::size_t>(height) > file.size() - data_offset)
+        return "BMP: raster is shorter than the header declares";
+    out.width = static_cast<int>(width);
+    out.height = static_cast<int>(height);
+    out.rgb.resize(static_cast<std::size_t>(width) * height * 3);
+    for (long long j = 0; j < height; ++j) {
+        const unsigned char* row = &file[data_offset + static_cast<std::size_t>(j) * row_bytes];
+        float* to = &out.rgb[static_cast<std::size_t>(top_down ? j : height - 1 - j) * width * 3];
+        for (long long x = 0; x < width; ++x, to += 3) {
+            if (bits <= 8) {
+                const std::size_t bit = static_cast<std::size_t>(x) * bits;
+                const std::size_t index = (row[bit >> 3] >> (8 - bits - (bit & 7))) & ((1u << bits) - 1);
+                if (index >= entries) return "BMP: colour index out of range";
+                for (int c = 0; c < 3; ++c) to[c] = table[index * entry_bytes + 2 - c] / 255.0f;  // stored blue, green, red
+            } else if (bits == 24) {
+                for (int c = 0; c < 3; ++c) to[c] = row[3 * x + 2 - c] / 255.0f;
+            } else {
+                const std::uint32_t value = bits == 16 ? le16(row + 2 * x) : le32(row + 4 * x);
+                for (int c = 0; c < 3; ++c) to[c] = masked_field(value, mask[c]);
+            }
+        }
+    }
+    return "";
+}
+
 bool ends_with(const std::string& s, const char* suffix) {
     const std::size_t n = std::strlen(suffix);
     if (s.size() < n) return false;
@@ -291,7 +380,8 @@ std::string load_image(const std::string& path, Image& out) {
     if (file.size() >= 8 && !std::memcmp(file.data(), kPngSignature, 8)) return decode_png(file, out);
     if (file.size() >= 3 && file[0] == 'P' && (file[1] == '6' || file[1] == '5')) return decode_netpbm(file, out);
     if (file.size() >= 2 && file[0] == 0xFF && file[1] == 0xD8) return decode_jpeg(file, out);
-    return path + " is neither a PNG, a JPEG nor a binary PPM/PGM file";
+    if (file.size() >= 2 && file[0] == 'B' && file[1] == 'M') return decode_bmp(file, out);
+    return path + " is neither a PNG, a JPEG, a BMP nor a binary PPM/PGM file";
 }
 
 namespace {

@@ -20,8 +20,8 @@ struct Image {
 };
 
 // Reads a PNG (any bit depth and colour type, interlaced or not), a JPEG
-// (Huffman-coded, sequential or progressive, grey or colour) or a binary PPM/PGM
-// (P6/P5), told apart by their first bytes.  Grey becomes R = G = B, alpha is
+// (Huffman-coded, sequential or progressive, grey or colour), an uncompressed
+// BMP or a binary PPM/PGM (P6/P5), told apart by their first bytes.  Grey becomes R = G = B, alpha is
 // dropped, samples are divided by their maximum value (image_utils.cpp:27-30
 // divides bytes by 255).  Returns "" or the reason for failure.
 std::string load_image(const std::string& path, Image& out);
