@@ -42,12 +42,14 @@ def _check(gpu, depth):
     np.testing.assert_array_equal(rank, inverse)
 
 
-@pytest.mark.parametrize("n", [1, 2, 63, 64, 65, 511, 512, 513, 2047, 2048, 2049, 4096, 10_000, 200_000, 1_000_003])
+# (up to 4096 keys one block sorts alone, with 2 or 4 keys per lane; above, tiles of 4096 keys)
+@pytest.mark.parametrize("n", [1, 2, 63, 64, 65, 511, 512, 513, 1024, 1025, 2047, 2048, 2049, 4096, 4097, 8192, 8193, 10_000, 12_287,
+                               12_288, 12_289, 16_384, 200_000, 1_000_003])
 def test_uniform_depths(gpu, n):
     _check(gpu, np.random.default_rng(n).uniform(0.0, 1.0, n))
 
 
-@pytest.mark.parametrize("n", [5, 2048, 50_000, 300_001])
+@pytest.mark.parametrize("n", [5, 2048, 9000, 50_000, 300_001])
 def test_ties_keep_index_order(gpu, n):
     r = np.random.default_rng(n)
     _check(gpu, r.integers(0, 4, n).astype(np.float32) * 0.25)  # four distinct depths
@@ -86,7 +88,7 @@ def test_nans_sort_by_their_bits(gpu):
     _check(gpu, d)
 
 
-@pytest.mark.parametrize("n", [4097, 123_457])
+@pytest.mark.parametrize("n", [700, 4097, 11_111, 123_457])
 def test_sorted_and_reversed_inputs(gpu, n):
     d = np.linspace(-1.0, 1.0, n).astype(np.float32)
     _check(gpu, d)
@@ -96,10 +98,11 @@ def test_sorted_and_reversed_inputs(gpu, n):
 def test_every_byte_position_decides_somewhere(gpu):
     """Keys that differ in one byte only, for each of the four bytes a pass looks at."""
     base = np.uint32(0x3F000000)
-    for byte in range(4):
-        r = np.random.default_rng(byte)
-        bits = (base + (r.integers(0, 256 if byte < 3 else 64, 20_000).astype(np.uint32) << np.uint32(8 * byte))).astype(np.uint32)
-        _check(gpu, bits.view(np.float32))
+    for n in (20_000, 6_000):
+        for byte in range(4):
+            r = np.random.default_rng(byte)
+            bits = (base + (r.integers(0, 256 if byte < 3 else 64, n).astype(np.uint32) << np.uint32(8 * byte))).astype(np.uint32)
+            _check(gpu, bits.view(np.float32))
 
 
 def test_calls_in_a_row_share_nothing(gpu):
